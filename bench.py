@@ -493,7 +493,13 @@ def main():
                          "model of equal size (pipeinfer_amd/tools/hybrid_bench.py); one JSON line per size")
     ap.add_argument("--compare-parallel", nargs="?", const="w1024,w2048,w4096", default=None, metavar="SIZES",
                     help="instead of the default workload: the same measurements for the Vikarax design (parallel mixer, gated experts) beside the Fasovik design at equal sizes; one JSON line per size")
+    ap.add_argument("--compare-postnorm", nargs="?", const="w1024,w2048,w4096", default=None, metavar="SIZES",
+                    help="instead of the default workload: the same measurements for the Rafusun design (delta-rule and attention + time-mix layers, the norm after the sum) beside the Vikarax design "
+                         "with a dense feed-forward at equal sizes; one JSON line per size")
     args = ap.parse_args()
+    if args.compare_postnorm:
+        from pipeinfer_amd.tools import hybrid_bench
+        return hybrid_bench.main_postnorm(args.compare_postnorm.split(","), args.cache)
     if args.compare_parallel:
         from pipeinfer_amd.tools import hybrid_bench
         return hybrid_bench.main_parallel(args.compare_parallel.split(","), args.cache)

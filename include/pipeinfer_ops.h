@@ -177,7 +177,7 @@ PI_API int pi_op_topk(const float * logits_dev, int n_vocab, int n_tok, int k, i
 /* ---- dense bfloat16 matrices and the operators of hybrid blocks (recurrent / low-rank-attention mixers, routed feed-forwards) --------------------------------------
  * Weights are PI_BF16 pi_weights ([rows][K] as stored, pi_weight_upload(PI_BF16, K, rows, ...)); activations, norms, scores, states and outputs are fp32.
  * exact = 0: activations are rounded to bfloat16 where they enter a matrix product (fp32 accumulation); exact = 1: nothing is rounded, every product is an fp32 fma. */
-enum pi_act { PI_ACT_NONE = 0, PI_ACT_SILU = 1, PI_ACT_SIGMOID = 2, PI_ACT_RELU_SQR = 3 };
+enum pi_act { PI_ACT_NONE = 0, PI_ACT_SILU = 1, PI_ACT_SIGMOID = 2, PI_ACT_RELU_SQR = 3, PI_ACT_TANH = 4, PI_ACT_GELU_TANH = 5 /* 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))) */ };
 /* out[t][:] = widen(table[tokens[t]]) * scale */
 PI_API int pi_op_embed(const pi_weight * table, const int32_t * tokens_dev, int n_tok, float scale, float * out_dev, void * stream);
 /* out[t][r] = act(W[r] . x[t]); rows [0, rows_a) take act_a, the others act_b (projections that share their input are one matrix and one launch); strides in floats */
@@ -274,6 +274,43 @@ PI_API int pi_op_moe_experts_grouped_act(const pi_weight * w_up, const pi_weight
 /* pi_op_moe_experts with the expert's activation as a parameter: glu = 0: relu(W_up x)^2; glu = 1: w_up holds [gate (ff rows) | up (ff rows)] per expert and the hidden values are silu(gate) * up */
 PI_API int pi_op_moe_experts_act(const pi_weight * w_up, const pi_weight * w_down, int n_exp, int ff, int glu, const float * x_dev, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,
                                  int exact, float * up_dev, float * out_dev, int64_t out_stride, void * stream);
+
+/* ---- operators of blocks whose norm comes after the sum, of recurrences with a decay per key channel, and of soft-max attention inside chunks -------------------------------- */
+/* out[t][:] = widen(table[tokens[t]]) * scale + widen(table2[rows2[t]]) (a row outside its table counts as zeros) */
+PI_API int pi_op_embed_pair(const pi_weight * table, const int32_t * tokens_dev, int n_tok, float scale, const pi_weight * table2, const int32_t * rows2_dev, float * out_dev, void * stream);
+/* the end of a sublayer, R(y) = y / sqrt(mean(y^2) + eps):  m = b ? mean_mult * (R(a) * wa + R(b) * wb) : a;  out = R(alpha * x + layer_scale * m) * w  (layer_scale nullable: 1);
+ * w_next != NULL: out_next = R(out) * w_next (the norm of whatever reads the stream next).  out may be x.  Rows of at most 8192 values */
+PI_API int pi_op_rms_post(const float * a_dev, int64_t a_stride, const float * wa_dev, const float * b_dev, int64_t b_stride, const float * wb_dev, float mean_mult, const float * layer_scale_dev,
+                          const float * x_dev, int64_t x_stride, float alpha, const float * w_dev, float eps, int n, int n_tok, float * out_dev, int64_t out_stride, const float * w_next_dev, float * out_next_dev,
+                          int64_t out_next_stride, void * stream);
+/* out[t][s][:] = h[t] + (h_prev - h[t]) * mu[s], s < n_mix (rows out_stride >= n_mix * n floats apart); h_prev: the sequence's previous token — the row before inside the pass, state_dev [slots][n] at a
+ * sequence's first token of the pass (zeros on a fresh slot); the sequence's last token of the pass becomes its state.  rec_dev as for pi_op_linear_attention */
+PI_API int pi_op_token_shift(const float * h_dev, int64_t h_stride, int n, const float * mu_dev, int n_mix, float * state_dev, const int32_t * rec_dev, int n_tok, float * out_dev, int64_t out_stride, void * stream);
+/* Recurrence over a [dim][vdim] state per head and sequence with a decay g[t][h][i] per token and key channel (state_dev [slots][heads][dim][vdim], rec_dev as for pi_op_linear_attention):
+ *   PI_RULE_DELTA  S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q              beta[t][h] = sigmoid(beta_raw) (nullable: 1)
+ *   PI_RULE_BONUS  o = (S + diag(bonus_h) k v^T)^T q;  S <- diag(g) S + k v^T                       bonus_dev [heads][dim] (nullable: 0)
+ * decay_mode 0: g = decay_raw; 1: g = exp(-exp(decay_raw + decay_bias[h][i])); 2: g = exp(-exp(a_log[h]) * softplus(decay_raw + decay_bias[h][i])).  qk_unit: q and k are divided by their length
+ * (sqrt(sum of squares + 1e-6)) per head first; q is then multiplied by q_mult.  q / k: [n_tok][qk_heads * dim] (head h reads q / k head h / (heads / qk_heads)), v: [n_tok][heads * vdim] */
+enum pi_recurrence_rule { PI_RULE_DELTA = 0, PI_RULE_BONUS = 1 };
+PI_API int pi_op_channel_recurrence(int rule, const float * q_dev, int64_t q_stride, const float * k_dev, int64_t k_stride, const float * v_dev, int64_t v_stride, const float * decay_raw_dev, int64_t decay_stride,
+                                    int decay_mode, const float * decay_bias_dev, const float * a_log_dev, const float * beta_raw_dev, int64_t beta_stride, const float * bonus_dev, int qk_unit, float q_mult,
+                                    int heads, int qk_heads, int dim, int vdim, float * state_dev, const int32_t * rec_dev, int n_tok, int max_segments, float * out_dev, int64_t out_stride, void * stream);
+PI_API int pi_op_channel_recurrence_reserve(void);                 /* once per process, outside graph capture: the LDS limit wide keys need */
+/* out[t][h][i] = y[t][h][i] / sqrt(mean_i(y[t][h]^2) + eps) * w[(w_per_head ? h * n : 0) + i] * act(gate[t][h][i]) (gate nullable; gate_act PI_ACT_NONE, _SIGMOID or _SILU); out may be y */
+PI_API int pi_op_head_norm_gate(const float * y_dev, int64_t y_stride, int heads, int n, const float * w_dev, int w_per_head, const float * gate_dev, int64_t gate_stride, int gate_act, float eps, int n_tok,
+                                float * out_dev, int64_t out_stride, void * stream);
+/* pi_op_qkv_prepare with its order and pairing as parameters: norm_first != 0: R(.) * w then the rotation, else the rotation first and R(.) * w over the rotated head (weights nullable: 1);
+ * pairing: dimension i with i + dims / 2, or 2i with 2i + 1; v_norm = 0: value heads are cached as they are */
+enum pi_rot_pairing { PI_PAIR_HALVES = 0, PI_PAIR_NEIGHBOURS = 1 };
+PI_API int pi_op_qkv_prepare_ex(const float * q_dev, const float * k_dev, const float * v_dev, int64_t stride, const float * q_norm_w, const float * k_norm_w, float eps, int heads, int kv_heads, int dim, int vdim,
+                                const void * rotary_table, int norm_first, int pairing, int v_norm, const int32_t * pos_dev, int n_tok, float * q_out_dev, int64_t q_out_stride, float * k_cache_dev, float * v_cache_dev,
+                                int32_t * cell_pos_dev, const int32_t * dyn_dev, void * stream);
+/* pi_op_chunk_attention with the kind of weights as a parameter.  s = q . k * scale + head_bias[h], softcap > 0: s <- softcap * tanh(s / softcap) (soft-max kinds);
+ * PI_WEIGHTS_SIGMOID: sigmoid(s), nothing normalised; PI_WEIGHTS_SOFTMAX: exp(s) / sum exp(s) over the visible cells; PI_WEIGHTS_SOFTMAX_SINK: exp(s) / (1 + sum exp(s)) */
+enum pi_attention_weights { PI_WEIGHTS_SIGMOID = 0, PI_WEIGHTS_SOFTMAX = 1, PI_WEIGHTS_SOFTMAX_SINK = 2 };
+PI_API int pi_op_chunk_attention_ex(const float * q_dev, int64_t q_stride, const float * k_cache_dev, const float * v_cache_dev, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
+                                    const float * head_bias_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int weights, float softcap, int chunk, int heads, int kv_heads,
+                                    int dim, int vdim, int n_tok, int n_kv, float * out_dev, int64_t out_stride, const int32_t * dyn_dev, void * stream);
 
 #ifdef __cplusplus
 }

@@ -42,7 +42,7 @@ llama_context::~llama_context() {
     if (hop_host) (void) hipHostFree(hop_host);
     pi_free(hop_dev);
     pi_free(abort_dev);
-    void * bufs[] = { cell_pos, hist, h_out2, ssd_dt, lat_cache, rec_state, rec_dev, h_in, h_att, h_out, moe_w, moe_up, moe_dn, lat_scratch, rec_scratch, moe_sel, moe_idx, k_cache, v_cache, x, x2, nx, nx2, qkv, att, up, gate, logits_dev, q16, q8a, q8b, q8c, tokens_dev, pos_dev, dyn_dev, mask_dev, topk_ids_dev, topk_vals_dev, topk_sum_dev, topk_scratch_dev };
+    void * bufs[] = { cell_pos, hist, h_out2, ssd_dt, lat_cache, rec_state, rec_dev, pair_dev, h_in, h_att, h_out, moe_w, moe_up, moe_dn, lat_scratch, rec_scratch, moe_sel, moe_idx, k_cache, v_cache, x, x2, nx, nx2, qkv, att, up, gate, logits_dev, q16, q8a, q8b, q8c, tokens_dev, pos_dev, dyn_dev, mask_dev, topk_ids_dev, topk_vals_dev, topk_sum_dev, topk_scratch_dev };
     for (void * b : bufs) pi_free(b);
     if (rope) pi_rope_table_free(rope);
     if (stream) (void) hipStreamDestroy(stream);
@@ -106,9 +106,25 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
     const int nb = ctx->n_batch, width = hp.n_embd;
     size_t lat = 0, rec = 0, in_w = 1, att_w = 1, up_w = 1, sel_w = 1, idx_n = 1, step_w = 0; bool positions = false;
     ctx->lat_off.assign(hp.hybrid.size(), 0); ctx->rec_off.assign(hp.hybrid.size(), 0);
-    if (hp.n_recurrent() > 0) ctx->slots.reset(new state_slots(std::max(1, ctx->n_state_slots)));
+    if (hp.n_recurrent() > 0 || hp.pair_buckets > 0) ctx->slots.reset(new state_slots(std::max(1, ctx->n_state_slots)));      // (the previous token of a pair embedding is per-sequence state as well)
     for (size_t i = 0; i < hp.hybrid.size(); i++) {
         const pi_hybrid_layer & H = hp.hybrid[i];
+        if (H.mixer == PI_MIXER_CHANNEL_DELTA || H.mixer == PI_MIXER_PARALLEL_SHIFT) {        // scratch rows as forward_post_norm_blocks lays them out
+            if (H.mixer == PI_MIXER_CHANNEL_DELTA) {
+                const pi_channel_delta & D = H.delta;
+                in_w = std::max(in_w, (size_t) D.in_rows());
+                att_w = std::max(att_w, (size_t) D.channels() + (size_t) D.heads * D.dim + (size_t) 2 * D.heads * D.vdim);
+            } else {
+                const pi_gate_attention & A = H.left; const pi_time_mix & R = H.shift;
+                ctx->lat_off[i] = lat; lat += (size_t) ctx->n_ctx * H.cell_floats();
+                in_w = std::max(in_w, (size_t) A.in_rows() + (size_t) 5 * width);
+                att_w = std::max(att_w, (size_t) A.heads * (A.dim + A.vdim) + (size_t) 7 * R.inner() + (size_t) R.decay_rank);
+                positions = true;
+            }
+            ctx->rec_off[i] = rec; rec += (size_t) ctx->slots->size() * H.state_floats();
+            if (H.has_mlp) in_w = std::max(in_w, (size_t) 3 * H.ff);
+            continue;
+        }
         if (H.mixer == PI_MIXER_PARALLEL) {                                  // keys | values per cell; the recurrence's matrix and the convolution's last inputs per sequence
             const pi_gate_attention & A = H.left; const pi_ssd & R = H.right;
             ctx->lat_off[i] = lat; lat += (size_t) ctx->n_ctx * H.cell_floats();
@@ -140,7 +156,7 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
     }
     if (!(ctx->x = (float *) dev((size_t) 4 * nb * width)) || !(ctx->nx = (float *) dev((size_t) 4 * nb * width)) || !(ctx->h_out = (float *) dev((size_t) 4 * nb * width)) ||
         !(ctx->h_in = (float *) dev((size_t) 4 * nb * in_w)) || !(ctx->h_att = (float *) dev((size_t) 4 * nb * att_w)) || !(ctx->moe_up = (float *) dev((size_t) 4 * nb * up_w)) ||
-        !(ctx->moe_w = (float *) dev((size_t) 4 * nb * sel_w)) || !(ctx->moe_dn = (float *) dev((size_t) 4 * nb * sel_w * width)) || !(ctx->moe_idx = (int32_t *) dev((size_t) 4 * idx_n)) || !(ctx->moe_sel = (int32_t *) dev((size_t) 4 * nb * sel_w)) || (ctx->slots && !(ctx->rec_dev = (int32_t *) dev((size_t) 4 * nb))) ||
+        !(ctx->moe_w = (float *) dev((size_t) 4 * nb * sel_w)) || !(ctx->moe_dn = (float *) dev((size_t) 4 * nb * sel_w * width)) || !(ctx->moe_idx = (int32_t *) dev((size_t) 4 * idx_n)) || !(ctx->moe_sel = (int32_t *) dev((size_t) 4 * nb * sel_w)) || (ctx->slots && !(ctx->rec_dev = (int32_t *) dev((size_t) 4 * nb))) || (hp.pair_buckets > 0 && !(ctx->pair_dev = (int32_t *) dev((size_t) 4 * nb))) ||
         !(ctx->tokens_dev = (int32_t *) dev((size_t) 4 * nb)) || !(ctx->pos_dev = (int32_t *) dev((size_t) 4 * nb)) || !(ctx->dyn_dev = (int32_t *) dev((size_t) 4 * (4 + 2 * nb))))
         return false;
     {   // abort word + cancel flags + the control stream cancels travel on
@@ -151,7 +167,7 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
         if (hipStreamCreateWithFlags(&ctx->ctl_stream, hipStreamNonBlocking) != hipSuccess) { err = "hipStreamCreate(control) failed"; return false; }
     }
     ctx->use_graphs = ctx->use_graphs && getenv("PI_NO_GRAPHS") == nullptr;
-    if (pi_op_latent_attention_reserve() != 0 || (hp.n_recurrent() > 0 && pi_op_linear_attention_reserve() != 0)) { err = pi_last_error(); return false; }
+    if (pi_op_latent_attention_reserve() != 0 || (hp.n_recurrent() > 0 && (pi_op_linear_attention_reserve() != 0 || pi_op_channel_recurrence_reserve() != 0))) { err = pi_last_error(); return false; }
     ctx->mask_cap_words = (size_t) nb * ((ctx->n_ctx + 31) / 32);
     if (!(ctx->mask_dev = (uint32_t *) dev(ctx->mask_cap_words * 4))) return false;
     if (!(ctx->logits_dev = (float *) dev((size_t) 4 * nb * hp.n_vocab)) || !(ctx->topk_ids_dev = (int32_t *) dev((size_t) 4 * nb * 8)) ||
@@ -395,10 +411,92 @@ static bool forward_pre_post_blocks(llama_context * ctx, int n_tok, int n_kv) {
     return true;
 }
 
+// Blocks whose norm comes after the sum (hp.post_norm), R(y) = y / sqrt(mean(y^2) + eps):   x <- R(alpha x + ls1 * mixer(x)) * w1;   x <- R(alpha x + ls2 * ff(x)) * w2.   The sublayers read x itself.
+//   channel delta    ONE projection [q | k | v | a1 | g1 | beta] -> convolution + silu over q | k | v (+ its state) -> the second halves of the low-rank decay and gate projections -> the recurrence
+//                    (unit q / k, sigmoid(beta), the decays formed from their raw values inside the kernel) -> per-head norm * weight * sigmoid(gate) -> output projection
+//   attention + time mix   [q | k | v] -> rotation in neighbouring pairs, then R(.) per head, cache store -> chunked soft-max attention with a sink and capped scores -> W_o;
+//                    token shift (five mixes of the token and the one before it, + its state) -> r, k, v, silu(g), tanh(w1) from their own mixes -> w2 -> the recurrence with a bonus for the token
+//                    itself (decays exp(-exp(. + w0)) formed inside) -> per-head norm * weight * gate -> W_o;   the mixer's result = (R(left) * w_l + R(right) * w_r) / 2, formed by the row kernel
+// Every sublayer ends in ONE row kernel (pi_op_rms_post): [mean of the two normed branches ->] layer scale -> + alpha x -> norm [-> the model's final norm behind the last sublayer].
+static bool forward_post_norm_blocks(llama_context * ctx, int n_tok, int n_kv) {
+    llama_model * m = ctx->model;
+    const pi_hparams & hp = m->hparams;
+    hipStream_t s = ctx->stream;
+    const int width = hp.n_embd, ex = ctx->exact, nb = ctx->n_batch, n_slots = ctx->slots->size();
+    const float eps = hp.f_norm_rms_eps, alpha = hp.post_alpha;
+    const size_t n_layer = hp.hybrid.size();
+    float * x = ctx->x, * P = ctx->h_in, * A = ctx->h_att, * Y = ctx->h_out, * Y2 = ctx->h_out2;
+    if (m->pair_embd) OP_OK(pi_op_embed_pair(m->tok_embd, ctx->tokens_dev, n_tok, hp.embed_scale, m->pair_embd, ctx->pair_dev, x, s));
+    else OP_OK(pi_op_embed(m->tok_embd, ctx->tokens_dev, n_tok, hp.embed_scale, x, s));
+    for (size_t il = 0; il < n_layer; il++) {
+        const pi_hybrid_layer & H = hp.hybrid[il];
+        const pi_hybrid_weights & W = m->hweights[(size_t) H.weights];
+        const bool last_sub_is_mixer = il + 1 == n_layer && !H.has_mlp;
+        const float * ya = Y, * yb = nullptr;
+        if (H.mixer == PI_MIXER_CHANNEL_DELTA) {
+            const pi_channel_delta & D = H.delta;
+            const int64_t pw = D.in_rows(), gd = (int64_t) D.kv_heads * D.dim, hd = (int64_t) D.heads * D.dim, hv = (int64_t) D.heads * D.vdim, ch = D.channels();
+            float * C = A, * A2 = C + (size_t) nb * ch, * G2 = A2 + (size_t) nb * hd, * O = G2 + (size_t) nb * hv;
+            float * S = ctx->rec_state + ctx->rec_off[il], * conv_state = S + (size_t) n_slots * D.matrix_floats();
+            OP_OK(pi_op_dense(W.w_in, x, width, n_tok, P, pw, PI_ACT_NONE, pw, PI_ACT_NONE, ex, s));
+            OP_OK(pi_op_causal_conv(P, pw, (int) ch, D.conv, W.conv_w, nullptr, conv_state, ctx->rec_dev, n_tok, PI_ACT_SILU, C, ch, s));
+            OP_OK(pi_op_dense(W.w_a2, P + ch, pw, n_tok, A2, hd, PI_ACT_NONE, hd, PI_ACT_NONE, ex, s));
+            OP_OK(pi_op_dense(W.w_g2, P + ch + D.decay_rank, pw, n_tok, G2, hv, PI_ACT_NONE, hv, PI_ACT_NONE, ex, s));
+            OP_OK(pi_op_channel_recurrence(PI_RULE_DELTA, C, ch, C + gd, ch, C + 2 * gd, ch, A2, hd, 2, W.dt_bias, W.a_log, P + ch + D.decay_rank + D.gate_rank, pw, nullptr, 1, 1.0f / sqrtf((float) D.dim), D.heads, D.kv_heads, D.dim, D.vdim,
+                                           S, ctx->rec_dev, n_tok, n_slots, O, hv, s));
+            trace(ctx, "rec", (int) il, O, hv, n_tok);
+            OP_OK(pi_op_head_norm_gate(O, hv, D.heads, D.vdim, W.mix_norm, 0, G2, hv, PI_ACT_SIGMOID, eps, n_tok, O, hv, s));
+            OP_OK(pi_op_dense(W.w_o, O, hv, n_tok, Y, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
+        } else if (H.mixer == PI_MIXER_PARALLEL_SHIFT) {
+            const pi_gate_attention & L = H.left; const pi_time_mix & R = H.shift;
+            const int64_t pw = L.in_rows(), hd = (int64_t) L.heads * L.dim, hv = (int64_t) L.heads * L.vdim, gd = (int64_t) L.kv_heads * L.dim, inner = R.inner(), mw = (int64_t) 5 * width;
+            float * M = P + (size_t) nb * pw;                                                          // the five mixes [r | k | v | g | w] of every token
+            float * Q = A, * O = Q + (size_t) nb * hd, * RK = O + (size_t) nb * hv, * W1 = RK + (size_t) nb * 4 * inner, * WD = W1 + (size_t) nb * R.decay_rank, * O2 = WD + (size_t) nb * inner;
+            float * kc = ctx->lat_cache + ctx->lat_off[il], * vc = kc + (size_t) ctx->n_ctx * gd;
+            float * S = ctx->rec_state + ctx->rec_off[il], * shift_state = S + (size_t) n_slots * R.matrix_floats();
+            // attention branch
+            OP_OK(pi_op_dense(W.w_in, x, width, n_tok, P, pw, PI_ACT_NONE, pw, PI_ACT_NONE, ex, s));
+            OP_OK(pi_op_qkv_prepare_ex(P, P + hd, P + hd + gd, pw, nullptr, nullptr, eps, L.heads, L.kv_heads, L.dim, L.vdim, W.rotary, 0, PI_PAIR_NEIGHBOURS, 0, ctx->pos_dev, n_tok, Q, hd, kc, vc, ctx->cell_pos, ctx->dyn_dev, s));
+            OP_OK(pi_op_chunk_attention_ex(Q, hd, kc, vc, ctx->cell_pos, ctx->mask_dev, ctx->pos_dev, nullptr, nullptr, 0, PI_ACT_NONE, L.scale, 1.0f, L.weights, L.softcap, L.chunk, L.heads, L.kv_heads, L.dim, L.vdim, n_tok, n_kv,
+                                           O, hv, ctx->dyn_dev, s));
+            trace(ctx, "att", (int) il, O, hv, n_tok);
+            OP_OK(pi_op_dense(W.w_o, O, hv, n_tok, Y, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
+            // time-mix branch
+            OP_OK(pi_op_token_shift(x, width, width, W.mu, 5, shift_state, ctx->rec_dev, n_tok, M, mw, s));
+            OP_OK(pi_op_dense(W.w_r, M, mw, n_tok, RK, 4 * inner, PI_ACT_NONE, inner, PI_ACT_NONE, ex, s));
+            OP_OK(pi_op_dense(W.w_k, M + width, mw, n_tok, RK + inner, 4 * inner, PI_ACT_NONE, inner, PI_ACT_NONE, ex, s));
+            OP_OK(pi_op_dense(W.w_v, M + 2 * width, mw, n_tok, RK + 2 * inner, 4 * inner, PI_ACT_NONE, inner, PI_ACT_NONE, ex, s));
+            OP_OK(pi_op_dense(W.w_g, M + 3 * width, mw, n_tok, RK + 3 * inner, 4 * inner, PI_ACT_SILU, inner, PI_ACT_SILU, ex, s));
+            OP_OK(pi_op_dense(W.w_w1, M + 4 * width, mw, n_tok, W1, R.decay_rank, PI_ACT_TANH, R.decay_rank, PI_ACT_TANH, ex, s));
+            OP_OK(pi_op_dense(W.w_w2, W1, R.decay_rank, n_tok, WD, inner, PI_ACT_NONE, inner, PI_ACT_NONE, ex, s));
+            OP_OK(pi_op_channel_recurrence(PI_RULE_BONUS, RK, 4 * inner, RK + inner, 4 * inner, RK + 2 * inner, 4 * inner, WD, inner, 1, W.w0, nullptr, nullptr, 0, W.bonus, 0, 1.0f, R.heads, R.heads, R.dim, R.dim,
+                                           S, ctx->rec_dev, n_tok, n_slots, O2, inner, s));
+            trace(ctx, "rec", (int) il, O2, inner, n_tok);
+            OP_OK(pi_op_head_norm_gate(O2, inner, R.heads, R.dim, W.mix_norm, 1, RK + 3 * inner, 4 * inner, PI_ACT_NONE, eps, n_tok, O2, inner, s));
+            OP_OK(pi_op_dense(W.w_o2, O2, inner, n_tok, Y2, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
+            yb = Y2;
+        } else { ctx->last_error = "blocks with the norm after the sum are built for the channel-delta and the attention + time-mix mixers"; return false; }
+        OP_OK(pi_op_rms_post(ya, width, W.left_out, yb, width, W.right_out, 0.5f, W.ls1, x, width, alpha, W.norm1, eps, width, n_tok, x, width, last_sub_is_mixer ? m->output_norm : nullptr, ctx->nx, width, s));
+        if (H.has_mlp) {
+            const int ff = H.ff;
+            float * G = P + (size_t) nb * 2 * ff;
+            OP_OK(pi_op_dense(W.ff_up, x, width, n_tok, P, 2 * ff, PI_ACT_GELU_TANH, ff, PI_ACT_NONE, ex, s));        // gelu(gate) | up
+            OP_OK(pi_op_glu_mul(P, 2 * ff, ff, n_tok, G, ff, s));
+            OP_OK(pi_op_dense(W.ff_down, G, ff, n_tok, Y, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
+            OP_OK(pi_op_rms_post(Y, width, nullptr, nullptr, 0, nullptr, 1.0f, W.ls2, x, width, alpha, W.norm2, eps, width, n_tok, x, width, il + 1 == n_layer ? m->output_norm : nullptr, ctx->nx, width, s));
+        }
+        trace(ctx, "lout", (int) il, x, width, n_tok);
+    }
+    OP_OK(pi_op_dense(m->output, ctx->nx, width, n_tok, ctx->logits_dev, hp.n_vocab, PI_ACT_NONE, hp.n_vocab, PI_ACT_NONE, ex, s));
+    OP_OK(pi_op_topk(ctx->logits_dev, hp.n_vocab, n_tok, 8, ctx->topk_ids_dev, ctx->topk_vals_dev, ctx->topk_sum_dev, ctx->topk_scratch_dev, s));
+    return true;
+}
+
 static bool forward_hybrid(llama_context * ctx, int n_tok, int n_kv) {
     llama_model * m = ctx->model;
     const pi_hparams & hp = m->hparams;
     if (hp.pre_post_norm) return forward_pre_post_blocks(ctx, n_tok, n_kv);
+    if (hp.post_norm) return forward_post_norm_blocks(ctx, n_tok, n_kv);
     hipStream_t s = ctx->stream;
     const int width = hp.n_embd, ex = ctx->exact;
     const float eps = hp.f_norm_rms_eps, rm = hp.residual_mult;
@@ -608,6 +706,7 @@ static bool launch_inputs(llama_context * ctx, int n_tokens, const void * meta, 
               hipMemcpyAsync(ctx->dyn_dev, h_dyn, 16 + 4 * n_table, hipMemcpyHostToDevice, s) == hipSuccess &&
               hipMemcpyAsync(ctx->mask_dev, h_mask, (size_t) 4 * n_tokens * words, hipMemcpyHostToDevice, s) == hipSuccess;
     if (ok && ctx->rec_dev) ok = hipMemcpyAsync(ctx->rec_dev, h_mask + (size_t) n_tokens * words, (size_t) 4 * n_tokens, hipMemcpyHostToDevice, s) == hipSuccess;     // (behind the mask rows: the state slot of every token)
+    if (ok && ctx->pair_dev) ok = hipMemcpyAsync(ctx->pair_dev, h_mask + (size_t) n_tokens * (words + 1), (size_t) 4 * n_tokens, hipMemcpyHostToDevice, s) == hipSuccess;     // (behind the slot words: every token's row of the pair-embedding table)
     if (ok && x_in) ok = hop_store(ctx->x, x_in, (size_t) 4 * n_tokens * ctx->model->hparams.n_embd, s);      // device (this stage's ring: a kernel) or host (staged transport: a copy)
     if (!ok) ctx->last_error = "H2D of batch metadata failed";
     return ok;
@@ -943,8 +1042,12 @@ pi_run * context_start(llama_context * ctx, const llama_batch & batch_in, int & 
     // consecutive in the batch (the recurrence walks them in order inside one workgroup).
     const bool recurrent = ctx->slots != nullptr;
     std::vector<int32_t> rec; std::vector<int> fresh_taken;
+    // models with a pair embedding: the table row of every token, from the token before it in its sequence (the slot remembers the last one of earlier runs)
+    const pi_hparams & hp0 = ctx->model->hparams;
+    const bool pairs = recurrent && hp0.pair_buckets > 0;
+    std::vector<int32_t> pair_rows; std::vector<std::pair<int, int>> last_before;       // (slot, its last token before this run: put back when the run cannot be started)
     if (recurrent) {
-        rec.resize((size_t) n_tokens);
+        rec.resize((size_t) n_tokens); if (pairs) pair_rows.resize((size_t) n_tokens);
         std::set<int> closed; int cur = -1, cur_slot = -1; bool bad = false, full = false;
         for (int i = 0; i < n_tokens && !bad && !full; i++) {
             if (n_seq_id[i] != 1) { bad = true; break; }
@@ -957,19 +1060,26 @@ pi_run * context_start(llama_context * ctx, const llama_batch & batch_in, int & 
                 const bool fresh = ctx->slots->take_fresh(cur_slot);
                 if (fresh) fresh_taken.push_back(cur_slot);
                 rec[(size_t) i] = cur_slot | (fresh ? (1 << 30) : 0);
+                if (pairs) { last_before.push_back({ cur_slot, ctx->slots->last_token(cur_slot) }); if (fresh) ctx->slots->set_last_token(cur_slot, -1); }
             } else rec[(size_t) i] = cur_slot;
+            if (pairs) {
+                const int prev = ctx->slots->last_token(cur_slot), tok = batch_in.token[i];
+                pair_rows[(size_t) i] = prev < 0 ? hp0.pair_buckets : (int32_t) (((int64_t) prev * hp0.pair_mul_prev + (int64_t) tok * hp0.pair_mul_cur) % hp0.pair_buckets);
+                ctx->slots->set_last_token(cur_slot, tok);
+            }
         }
         if (bad || full) {
             for (int sl : fresh_taken) ctx->slots->mark_fresh(sl);
+            for (auto it = last_before.rbegin(); it != last_before.rend(); ++it) ctx->slots->set_last_token(it->first, it->second);
             ctx->cells->release_cells(kv_head, n_tokens);
             if (bad) { ctx->last_error = "a model with recurrent layers takes tokens of ONE sequence each, a sequence's tokens next to each other in the batch"; return nullptr; }
             ctx->last_error = "no free state slot: " + std::to_string(ctx->slots->size()) + " sequences are live (pipeinfer_context_set_state_slots)"; rc = 1; return nullptr;
         }
     }
-    const size_t meta_bytes = (size_t) n_tokens * 8 + 16 + (size_t) n_tokens * words * 4 + (recurrent ? (size_t) n_tokens * 4 : 0);
+    const size_t meta_bytes = (size_t) n_tokens * 8 + 16 + (size_t) n_tokens * words * 4 + (recurrent ? (size_t) n_tokens * 4 : 0) + (pairs ? (size_t) n_tokens * 4 : 0);
     pi_run * run = acquire_run(ctx, n_tokens, meta_bytes);
     // (a run that cannot be started gives the cells find_slot just allotted back: nothing was or will be written to them)
-    auto give_back = [&]() { ctx->cells->release_cells(kv_head, n_tokens); for (int sl : fresh_taken) ctx->slots->mark_fresh(sl); };
+    auto give_back = [&]() { ctx->cells->release_cells(kv_head, n_tokens); for (int sl : fresh_taken) ctx->slots->mark_fresh(sl); for (auto it = last_before.rbegin(); it != last_before.rend(); ++it) ctx->slots->set_last_token(it->first, it->second); };
     if (!run) { ctx->last_error = "out of pinned host memory"; give_back(); return nullptr; }
     run->batch_id = batch_in.batch_id; run->n_tokens = n_tokens; run->t_start_us = time_us(); run->sink = nullptr;
     run->run_id = (++ctx->run_counter) & 0x3fffffff; run->kv_head = kv_head; run->n_kv = n_kv;
@@ -994,6 +1104,7 @@ pi_run * context_start(llama_context * ctx, const llama_batch & batch_in, int & 
     ctx->cells->build_mask(n_kv, n_tokens, pos, n_seq_id, seq_id, h_mask, words);
     ctx->cells->post_decode(n_tokens);
     if (recurrent) memcpy(h_mask + (size_t) n_tokens * words, rec.data(), (size_t) 4 * n_tokens);
+    if (pairs) memcpy(h_mask + (size_t) n_tokens * (words + 1), pair_rows.data(), (size_t) 4 * n_tokens);
 
     run->meta_bytes = meta_bytes;
     if (ctx->run_tap) ctx->run_tap(ctx->run_tap_user, run->run_id, run->batch_id, n_tokens, run->meta_host, meta_bytes, nullptr);

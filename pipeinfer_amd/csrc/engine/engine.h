@@ -33,7 +33,8 @@
 // LLAMA and FALCON have their own blocks in forward(); the others are one generic sequential block (norm -> attention -> + -> norm -> MLP -> +) described by pi_block below
 enum pi_arch { PI_ARCH_LLAMA = 0, PI_ARCH_FALCON = 1, PI_ARCH_BAICHUAN = 2, PI_ARCH_STARCODER = 3, PI_ARCH_REFACT = 4, PI_ARCH_BLOOM = 5, PI_ARCH_MPT = 6, PI_ARCH_STABLELM = 7, PI_ARCH_PERSIMMON = 8,
                PI_ARCH_FASOVIK = 9 /* a hybrid model: a list of layers, each with its own mixer (pi_hybrid_layer), read from config.json + model.safetensors */,
-               PI_ARCH_VIKARAX = 10 /* hybrid as well: layer norms before and after every sublayer, a learned average over depth, mixers of two parallel branches */ };
+               PI_ARCH_VIKARAX = 10 /* hybrid as well: layer norms before and after every sublayer, a learned average over depth, mixers of two parallel branches */,
+               PI_ARCH_RAFUSUN = 11 /* hybrid as well: the norm AFTER the sum (x <- R(alpha x + ls * sublayer(x)) * w), a hashed pair embedding, delta-rule and attention + time-mix mixers */ };
 
 // what the reference's build_* functions differ in (llama.cpp:3985-4104 baichuan, 4229-4327 starcoder, 4540-4630 refact, 4632-4725 bloom, 4727-4825 mpt, 4827-4939 stablelm)
 struct pi_block {
@@ -51,16 +52,28 @@ struct pi_block {
 // mixture of experts (or absent).  A layer may use another layer's tensors (`weights`) while keeping a cache / state of its own.
 enum pi_mixer_kind { PI_MIXER_LATENT_ATTENTION = 0,   // keys / values are up-projections of one cached low-rank latent, no positions, causal, soft-max with a per-head sink
                      PI_MIXER_LIGHTNING = 1,          // linear attention with a per-head decay: a [dim][vdim] state per head and sequence
-                     PI_MIXER_PARALLEL = 2 };         // two branches that read the same input, summed with fixed factors: chunked sigmoid attention (pi_gate_attention) + a selective recurrence (pi_ssd)
+                     PI_MIXER_PARALLEL = 2,           // two branches that read the same input, summed with fixed factors: chunked sigmoid attention (pi_gate_attention) + a selective recurrence (pi_ssd)
+                     PI_MIXER_CHANNEL_DELTA = 3,      // gated delta rule with a decay per key channel behind short convolutions (pi_channel_delta)
+                     PI_MIXER_PARALLEL_SHIFT = 4 };   // two branches, each RMS-normed over the width, averaged: chunked soft-max attention (pi_gate_attention) + time mixing with a token shift (pi_time_mix)
 // attention with grouped key / value heads, normed and partly rotated q / k, unit-norm values, un-normalised sigmoid weights inside chunks of positions, a per-head output gate
-struct pi_gate_attention { int heads = 0, kv_heads = 0, dim = 0, vdim = 0, rot_dims = 0, chunk = 0; float rot_base = 10000.0f, scale = 1.0f;
-                           int in_rows() const { return heads * dim + kv_heads * (dim + vdim) + heads; } };                      // [q | k | v | gate]
+// (weights / softcap / gated: the soft-max variants — pi_attention_weights — with a tanh cap on the scores and no output gate)
+struct pi_gate_attention { int heads = 0, kv_heads = 0, dim = 0, vdim = 0, rot_dims = 0, chunk = 0; float rot_base = 10000.0f, scale = 1.0f; int weights = PI_WEIGHTS_SIGMOID; float softcap = 0.0f; bool gated = true;
+                           int in_rows() const { return heads * dim + kv_heads * (dim + vdim) + (gated ? heads : 0); } };         // [q | k | v | gate]
 // selective state-space recurrence: a [state][vdim] matrix per head and sequence, B / C shared by the heads of a group, a causal convolution of `conv` taps over x, B, C
 struct pi_ssd { int heads = 0, vdim = 0, state = 0, groups = 0, conv = 0, norm_groups = 1;
                 int inner() const { return heads * vdim; } int channels() const { return inner() + 2 * groups * state; } int in_rows() const { return 2 * inner() + 2 * groups * state + heads; }   // [z | x | B | C | dt]
                 size_t state_floats() const { return (size_t) heads * state * vdim + (size_t) std::max(conv - 1, 0) * channels(); } };
+// gated delta rule: q, k (kv_heads x dim) and v (heads x vdim) through a causal convolution of `conv` taps and silu, q / k unit vectors, beta = sigmoid of a projection, a decay per head and key
+// channel from a projection of rank decay_rank, an output gate from one of rank gate_rank; per sequence a [dim][vdim] matrix per head and the convolution's last conv - 1 inputs
+struct pi_channel_delta { int heads = 0, kv_heads = 0, dim = 0, vdim = 0, conv = 0, decay_rank = 0, gate_rank = 0;
+                          int channels() const { return 2 * kv_heads * dim + heads * vdim; } int in_rows() const { return channels() + heads + decay_rank + gate_rank; }   // [q | k | v | a1 | g1 | beta]
+                          size_t matrix_floats() const { return (size_t) heads * dim * vdim; } size_t state_floats() const { return matrix_floats() + (size_t) std::max(conv - 1, 0) * channels(); } };
+// time mixing: r, k, v, gate and the decay each read their own mix of the token and the token before it; a decay per head and key channel from a projection of rank decay_rank, a bonus for the
+// token itself; per sequence a [dim][dim] matrix per head and the previous token's input (width values)
+struct pi_time_mix { int heads = 0, dim = 0, decay_rank = 0, width = 0;
+                     int inner() const { return heads * dim; } size_t matrix_floats() const { return (size_t) heads * dim * dim; } size_t state_floats() const { return matrix_floats() + (size_t) width; } };
 enum pi_mlp_kind { PI_MLP_NONE = 0, PI_MLP_MOE_RELU_SQR = 1 /* routed by a soft-max with correction, experts relu(up)^2, identity experts */, PI_MLP_DENSE_RELU_SQR = 2,
-                   PI_MLP_MOE_GLU = 3 /* routed by sigmoid scores inside the best groups, experts silu(gate) * up, an optional shared expert */ };
+                   PI_MLP_MOE_GLU = 3 /* routed by sigmoid scores inside the best groups, experts silu(gate) * up, an optional shared expert */, PI_MLP_DENSE_GEGLU = 4 /* down (gelu_tanh(gate) * up) */ };
 struct pi_hybrid_layer {
     pi_mixer_kind mixer = PI_MIXER_LATENT_ATTENTION;
     int weights = 0;                                  // index of the layer that owns the tensors (its own index unless shared)
@@ -68,13 +81,19 @@ struct pi_hybrid_layer {
     float scale = 1.0f;                               // latent attention: factor on q . k
     std::vector<float> decay;                         // lightning: per head
     pi_gate_attention left; pi_ssd right; float left_scale = 1.0f, right_scale = 1.0f;      // PI_MIXER_PARALLEL
+    pi_channel_delta delta; pi_time_mix shift;                                              // PI_MIXER_CHANNEL_DELTA; PI_MIXER_PARALLEL_SHIFT (beside `left`)
     bool has_mlp = false; int n_expert = 0, n_identity = 0, top = 0, ff = 0;
     pi_mlp_kind mlp = PI_MLP_NONE; int route_groups = 0, route_keep = 0, shared_ff = 0;     // (has_mlp <=> mlp != PI_MLP_NONE)
     int cache_index = -1, state_index = -1;           // ordinal among the layers that keep a per-cell cache / a recurrent state
-    int in_rows() const { return mixer == PI_MIXER_PARALLEL ? left.in_rows() + right.in_rows() : mixer == PI_MIXER_LIGHTNING ? 2 * heads * dim + 2 * heads * vdim : heads * dim + kv_rank; }     // rows of the fused input projection
-    int out_cols() const { return mixer == PI_MIXER_PARALLEL ? std::max(left.heads * left.vdim, right.inner()) : heads * vdim; }                                                   // widest input of an output projection
-    size_t cell_floats() const { return mixer == PI_MIXER_PARALLEL ? (size_t) left.kv_heads * (left.dim + left.vdim) : mixer == PI_MIXER_LATENT_ATTENTION ? (size_t) kv_rank : 0; }   // cached per cell
-    size_t state_floats() const { return mixer == PI_MIXER_PARALLEL ? right.state_floats() : mixer == PI_MIXER_LIGHTNING ? (size_t) heads * dim * vdim : 0; }                       // kept per sequence
+    int in_rows() const { return mixer == PI_MIXER_CHANNEL_DELTA ? delta.in_rows() : mixer == PI_MIXER_PARALLEL_SHIFT ? left.in_rows() : mixer == PI_MIXER_PARALLEL ? left.in_rows() + right.in_rows() : mixer == PI_MIXER_LIGHTNING ? 2 * heads * dim + 2 * heads * vdim : heads * dim + kv_rank; }     // rows of the fused input projection
+    int out_cols() const { return mixer == PI_MIXER_CHANNEL_DELTA ? delta.heads * delta.vdim : mixer == PI_MIXER_PARALLEL_SHIFT ? std::max(left.heads * left.vdim, shift.inner()) : mixer == PI_MIXER_PARALLEL ? std::max(left.heads * left.vdim, right.inner()) : heads * vdim; }                                                   // widest input of an output projection
+    size_t cell_floats() const { return mixer == PI_MIXER_CHANNEL_DELTA ? 0 : mixer == PI_MIXER_PARALLEL || mixer == PI_MIXER_PARALLEL_SHIFT ? (size_t) left.kv_heads * (left.dim + left.vdim) : mixer == PI_MIXER_LATENT_ATTENTION ? (size_t) kv_rank : 0; }   // cached per cell
+    size_t state_floats() const { return mixer == PI_MIXER_CHANNEL_DELTA ? delta.state_floats() : mixer == PI_MIXER_PARALLEL_SHIFT ? shift.state_floats() : mixer == PI_MIXER_PARALLEL ? right.state_floats() : mixer == PI_MIXER_LIGHTNING ? (size_t) heads * dim * vdim : 0; }                       // kept per sequence
+    // a layer's per-sequence state has up to two parts, each stored [slots][part]: the recurrence's matrices, then the convolution's last inputs / the previous token's input
+    void state_parts(size_t parts[2]) const {
+        parts[0] = mixer == PI_MIXER_CHANNEL_DELTA ? delta.matrix_floats() : mixer == PI_MIXER_PARALLEL_SHIFT ? shift.matrix_floats() : mixer == PI_MIXER_PARALLEL ? (size_t) right.heads * right.state * right.vdim : state_floats();
+        parts[1] = state_floats() - parts[0];
+    }
 };
 struct pi_hybrid_weights {                            // the tensors of a layer that owns some
     pi_weight * w_in = nullptr;                       // latent attention: [q | dkv], lightning: [q | k | v | g] (projections of the same input, one matrix)
@@ -85,6 +104,10 @@ struct pi_hybrid_weights {                            // the tensors of a layer 
     float * norm1_b = nullptr, * norm2_b = nullptr, * post1 = nullptr, * post1_b = nullptr, * post2 = nullptr, * post2_b = nullptr, * depth = nullptr;      // biases of the pre-norms, the post-norms, the depth average's factors
     float * q_norm = nullptr, * k_norm = nullptr, * head_bias = nullptr, * conv_w = nullptr, * conv_b = nullptr, * dt_bias = nullptr, * a_log = nullptr, * skip = nullptr;
     void * rotary = nullptr;                          // pi_rotary_table of the layer's (dims, base)
+    // post-norm blocks: layer scales; channel delta: w_in = rows [q | k | v | a1 | g1 | beta], the second halves of the low-rank decay / gate projections; attention + time mix: w_in = [q | k | v], w_o = the
+    // attention branch's, the time mix's own projections (each reads its own mix of the input), its shift factors [r | k | v | g | w][width], decay offset, bonus, and both branches' width-norms
+    float * ls1 = nullptr, * ls2 = nullptr, * mu = nullptr, * w0 = nullptr, * bonus = nullptr, * left_out = nullptr, * right_out = nullptr;
+    pi_weight * w_a2 = nullptr, * w_g2 = nullptr, * w_r = nullptr, * w_k = nullptr, * w_v = nullptr, * w_g = nullptr, * w_w1 = nullptr, * w_w2 = nullptr, * w_o2 = nullptr;
     bool loaded = false;
 };
 
@@ -99,7 +122,10 @@ struct pi_hparams {
     // what the hybrid architectures' blocks differ in: layer norms (weight, bias) before AND after every sublayer or an RMS norm (1 + w) on its output only; the stream that
     // goes on after a layer = a learned weighted sum of the embedding output and every layer's result so far; an output head of its own or the embedding table; tanh cap on the logits
     bool pre_post_norm = false, depth_average = false, own_head = false; float logit_softcap = 0.0f;
-    bool hybrid_arch() const { return arch == PI_ARCH_FASOVIK || arch == PI_ARCH_VIKARAX; }
+    // ... or the norm after the sum: x <- R(post_alpha * x + ls * sublayer(x)) * w.  pair_buckets > 0: the embedding adds row (previous token * pair_mul_prev + token * pair_mul_cur) mod pair_buckets
+    // of a second table (row pair_buckets for a sequence's first token); the previous token is part of a sequence's state (state_slots)
+    bool post_norm = false; float post_alpha = 1.0f; int pair_buckets = 0, pair_mul_prev = 0, pair_mul_cur = 0;
+    bool hybrid_arch() const { return arch == PI_ARCH_FASOVIK || arch == PI_ARCH_VIKARAX || arch == PI_ARCH_RAFUSUN; }
     int n_latent() const { int n = 0; for (const auto & l : hybrid) n += l.cache_index >= 0; return n; }
     int n_recurrent() const { int n = 0; for (const auto & l : hybrid) n += l.state_index >= 0; return n; }
     int head_dim() const { return n_embd / n_head; }
@@ -126,6 +152,7 @@ struct llama_model {
     std::string name, path;
     int device = 0;
     uint64_t n_elements = 0, n_bytes = 0;
+    pi_weight * pair_embd = nullptr;                                                               // hashed pair embedding [pair_buckets + 1][n_embd]
     pi_weight * tok_embd = nullptr, * output = nullptr, * pos_embd = nullptr;                 // pos_embd: StarCoder's learned positions (llama.cpp:4251-4255)
     float * output_norm = nullptr, * output_norm_b = nullptr, * tok_norm = nullptr, * tok_norm_b = nullptr;   // tok_norm: Bloom's LayerNorm on the embeddings (llama.cpp:4650-4654)
     float * alibi_slopes = nullptr;                                                              // f32 [n_head] on the device when block.alibi > 0
@@ -218,6 +245,7 @@ struct llama_context {
     float * hist = nullptr, * h_out2 = nullptr, * ssd_dt = nullptr;   // depth average: the stream after the embedding and after every layer [n_layer + 1][n_batch][width]; second branch output; step sizes | decays
     std::unique_ptr<pi::state_slots> slots; int n_state_slots = 8;
     int32_t * rec_dev = nullptr;                              // per token of the pass: state slot (| 1 << 30: start from zero)
+    int32_t * pair_dev = nullptr;                             // per token of the pass: its row of the pair-embedding table (models with pair_buckets > 0)
     int exact = 0;                                            // 1: dense operators keep fp32 activations (pipeinfer_context_set_precision)
     float * h_in = nullptr, * h_att = nullptr, * h_out = nullptr, * moe_w = nullptr, * moe_up = nullptr, * moe_dn = nullptr, * lat_scratch = nullptr, * rec_scratch = nullptr; size_t lat_scratch_floats = 0, rec_scratch_floats = 0; int32_t * moe_sel = nullptr, * moe_idx = nullptr;   // hybrid scratch
     void * rope = nullptr;

@@ -188,13 +188,14 @@ extern "C" void llama_kv_cache_seq_cp(struct llama_context * ctx, llama_seq_id a
             if (dst < 0) { ctx->last_error = "llama_kv_cache_seq_cp: no free state slot"; fprintf(stderr, "%s\n", ctx->last_error.str().c_str()); return; }
             (void) ctx->slots->take_fresh(dst);
             if (ctx->slots->is_fresh(src)) ctx->slots->mark_fresh(dst);
+            ctx->slots->set_last_token(dst, ctx->slots->last_token(src));
             const pi_hparams & hp = ctx->model->hparams;
             for (size_t i = 0; i < hp.hybrid.size(); i++) {
                 const pi_hybrid_layer & H = hp.hybrid[i];
                 if (H.state_index < 0) continue;
                 float * base = ctx->rec_state + ctx->rec_off[i];
                 // (a layer's per-sequence state may have several parts, each [slots][part]: the recurrence's matrix, the convolution's last inputs)
-                const size_t parts[2] = { H.mixer == PI_MIXER_PARALLEL ? (size_t) H.right.heads * H.right.state * H.right.vdim : H.state_floats(), H.mixer == PI_MIXER_PARALLEL ? H.state_floats() - (size_t) H.right.heads * H.right.state * H.right.vdim : 0 };
+                size_t parts[2]; H.state_parts(parts);
                 for (int k = 0; k < 2; k++) {
                     if (parts[k] && pi_op_copy_f32(base + parts[k] * (size_t) src, base + parts[k] * (size_t) dst, (int64_t) parts[k], ctx->stream) != 0) { ctx->last_error = std::string("llama_kv_cache_seq_cp: ") + pi_last_error(); return; }
                     base += parts[k] * (size_t) ctx->slots->size();

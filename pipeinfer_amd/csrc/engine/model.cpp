@@ -40,9 +40,11 @@ llama_model::~llama_model() {
         pi_weight_free(l.ffn_gate); pi_weight_free(l.ffn_down); pi_weight_free(l.ffn_up);
     }
     for (auto & w : hweights) { pi_weight_free(w.w_in); pi_weight_free(w.w_uk); pi_weight_free(w.w_uv); pi_weight_free(w.w_o); pi_weight_free(w.router); pi_weight_free(w.e_up); pi_weight_free(w.e_down);
-                                pi_weight_free(w.ff_up); pi_weight_free(w.ff_down); if (w.rotary) pi_rotary_table_free(w.rotary); }
+                                pi_weight_free(w.ff_up); pi_weight_free(w.ff_down);
+                                for (pi_weight * x : { w.w_a2, w.w_g2, w.w_r, w.w_k, w.w_v, w.w_g, w.w_w1, w.w_w2, w.w_o2 }) pi_weight_free(x);
+                                if (w.rotary) pi_rotary_table_free(w.rotary); }
     for (void * t : retired_tables) pi_rotary_table_free(t);
-    pi_weight_free(tok_embd); pi_weight_free(output); pi_weight_free(pos_embd);
+    pi_weight_free(tok_embd); pi_weight_free(output); pi_weight_free(pos_embd); pi_weight_free(pair_embd);
     for (void * p : f32_allocs) pi_free(p);
 }
 
@@ -188,6 +190,12 @@ size_t llama_model::stage_weight_bytes(int l0, int l1, bool first, bool last, in
         for (size_t i = 0; i < hparams.hybrid.size(); i++) {
             const pi_hybrid_layer & H = hparams.hybrid[i];
             const size_t w = (size_t) hparams.n_embd;
+            if (H.mixer == PI_MIXER_CHANNEL_DELTA || H.mixer == PI_MIXER_PARALLEL_SHIFT) {      // the projections (low-rank ones in both halves), the small vectors, the gated feed-forward
+                if (H.mixer == PI_MIXER_CHANNEL_DELTA) { const pi_channel_delta & D = H.delta; b += 2 * ((size_t) D.in_rows() + (size_t) D.heads * D.vdim) * w + 2 * (size_t) D.heads * (D.dim * D.decay_rank + D.vdim * D.gate_rank) + 4 * (size_t) D.channels() * D.conv; }
+                else { const pi_time_mix & R = H.shift; b += 2 * ((size_t) H.left.in_rows() + (size_t) H.left.heads * H.left.vdim + 5 * (size_t) R.inner() + R.decay_rank) * w + 2 * (size_t) R.inner() * R.decay_rank + 4 * 9 * w; }
+                b += 4 * 4 * w + (H.has_mlp ? 6 * (size_t) H.ff * w : 0);
+                continue;
+            }
             if (H.mixer == PI_MIXER_PARALLEL) {                                // both branches' projections, the norms' vectors, the feed-forward a token uses
                 b += 2 * (size_t) H.in_rows() * w + 2 * ((size_t) H.left.heads * H.left.vdim + H.right.inner()) * w + 4 * 8 * w;
                 if (H.mlp == PI_MLP_DENSE_RELU_SQR) b += 4 * (size_t) H.ff * w;
@@ -306,7 +314,7 @@ extern "C" enum llama_vocab_type llama_vocab_type(const struct llama_model * m) 
 extern "C" uint64_t llama_model_size(const struct llama_model * m) { return m->n_bytes; }
 extern "C" uint64_t llama_model_n_params(const struct llama_model * m) { return m->n_elements; }
 extern "C" int llama_model_desc(const struct llama_model * m, char * buf, size_t n) {
-    static const char * names[] = { "llama", "falcon", "baichuan", "starcoder", "refact", "bloom", "mpt", "stablelm", "persimmon", "fasovik", "vikarax" };
+    static const char * names[] = { "llama", "falcon", "baichuan", "starcoder", "refact", "bloom", "mpt", "stablelm", "persimmon", "fasovik", "vikarax", "rafusun" };
     return snprintf(buf, n, "%s %s", names[m->hparams.arch], m->name.c_str());
 }
 

@@ -9,6 +9,11 @@
 // mask.size }, right: { heads, vdim, state, groups, conv, norm_groups }, left_scale, right_scale }, mlp: null | { kind: "dense", ff } | { kind: "moe", expert.ff, router.experts /
 // top / groups.count / groups.keep, shared.ff } }.  Tensors: embed, head, final.norm (+ .b), l<i>.norm1 / norm1b / norm2 / norm2b (+ .b), l<i>.dwa, l<i>.mix.left.{q, k, v, q.norm,
 // k.norm, pb, g, o}, l<i>.mix.right.{in, conv, conv.b, dt_bias, A_log, D, norm, o}, l<i>.mlp.{up, down} or l<i>.mlp.{router, e<k>.{gate, up, down}, shared.{gate, up, down}}.
+//
+// Rafusun (same files, other keys): vocab, width, norm.eps, postln_alpha, embedding.scale, embedding.bigram.{buckets, mul_prev, mul_cur}, layers[]: { type: "channel_delta", mixer: { heads, kv_heads, dim, vdim, conv } }
+// or { type: "parallel", mixer: { left: { heads, kv_heads, dim, vdim, scale, softcap, rot.dims / rot.base, mask.size }, right: { heads, dim } } }, mlp: null | { kind: "dense", ff }.  The ranks of the low-rank
+// projections are the tensors' own.  Tensors: embed, bigram, head, final.norm, l<i>.norm1 / norm2, l<i>.ls1 / ls2, l<i>.mix.{q, k, v (+ .conv), b, A_log, dt_bias, a1, a2, g1, g2, norm, o} or
+// l<i>.mix.left.{q, k, v, o, out}, l<i>.mix.right.{mu.{r, k, v, g, w}, r, k, v, g, w1, w2, w0, u, norm, o, out}, l<i>.mlp.{gate, up, down}.
 #include "engine.h"
 #include "json.h"
 
@@ -88,6 +93,18 @@ struct loader {
         for (size_t i = 0; i < v.size(); i++) v[i] = bf16_to_f32(((const uint16_t *) t->data)[i]);
         return vector_f32(v);
     }
+    // several vectors (or [rows][cols] tables of equal cols) one after the other, widened to fp32
+    float * vectors(const std::vector<std::pair<std::string, int64_t>> & parts, int64_t cols) {
+        std::vector<float> v;
+        for (const auto & p : parts) {
+            const pi::st_tensor * t = cols > 0 ? get(p.first, { p.second, cols }) : get(p.first, { p.second });
+            if (!t) return nullptr;
+            const size_t n = (size_t) (p.second * std::max<int64_t>(cols, 1)), at = v.size();
+            v.resize(at + n);
+            for (size_t i = 0; i < n; i++) v[at + i] = bf16_to_f32(((const uint16_t *) t->data)[i]);
+        }
+        return vector_f32(v);
+    }
     float * vector(const std::string & name, int64_t n) {
         const pi::st_tensor * t = get(name, { n });
         if (!t) return nullptr;
@@ -162,6 +179,72 @@ static bool read_vikarax_config(const pi::json & cfg, pi_hparams & hp, std::stri
     return true;
 }
 
+// Rafusun: layers of two kinds (a delta-rule mixer, or attention beside time mixing), an optional gated dense feed-forward, the norm after the sum
+static bool read_rafusun_config(const pi::json & cfg, const pi::safetensors_file * st, pi_hparams & hp, std::string & what) {
+    using pi::json;
+    double d;
+    if (!num_at(cfg, "norm.eps", d)) { what = "no 'norm.eps'"; return false; }
+    hp.f_norm_eps = hp.f_norm_rms_eps = (float) d;
+    if (!num_at(cfg, "postln_alpha", d)) { what = "no 'postln_alpha'"; return false; }
+    hp.post_alpha = (float) d; hp.post_norm = hp.own_head = true;
+    hp.embed_scale = num_at(cfg, "embedding.scale", d) ? (float) d : 1.0f;
+    if (cfg.at("embedding.bigram") && !cfg.at("embedding.bigram")->is_null()) {
+        if (!int_at(cfg, "embedding.bigram.buckets", hp.pair_buckets) || !int_at(cfg, "embedding.bigram.mul_prev", hp.pair_mul_prev) || !int_at(cfg, "embedding.bigram.mul_cur", hp.pair_mul_cur) || hp.pair_buckets < 1) { what = "embedding.bigram needs a positive 'buckets', 'mul_prev' and 'mul_cur'"; return false; }
+    }
+    const json * layers = cfg.find("layers");
+    if (!layers || !layers->is_arr() || layers->arr.empty()) { what = "'layers' must be a non-empty list"; return false; }
+    hp.n_layer = (int) layers->arr.size();
+    hp.n_head = hp.n_head_kv = 1; hp.n_ctx_train = 0;
+    int n_cache = 0, n_state = 0;
+    // the rank of a low-rank projection is the first size of its first matrix [rank][width]
+    auto rank_of = [&](const std::string & name, int & out) { out = 0; if (!st) return true; const pi::st_tensor * t = st->tensor(name); if (!t || t->shape.size() != 2 || t->shape[0] < 1 || t->shape[1] != hp.n_embd) return false; out = (int) t->shape[0]; return true; };
+    for (int i = 0; i < hp.n_layer; i++) {
+        const json & jl = layers->arr[(size_t) i];
+        const std::string where = "layers[" + std::to_string(i) + "]: ", p = "l" + std::to_string(i) + ".mix.";
+        auto bad = [&](const std::string & w) { what = where + w; return false; };
+        pi_hybrid_layer H;
+        H.weights = i;
+        const json * type = jl.find("type");
+        if (!type || !type->is_str()) return bad("no 'type'");
+        if (type->str == "channel_delta") {
+            H.mixer = PI_MIXER_CHANNEL_DELTA;
+            pi_channel_delta & D = H.delta;
+            if (!int_at(jl, "mixer.heads", D.heads) || !int_at(jl, "mixer.kv_heads", D.kv_heads) || !int_at(jl, "mixer.dim", D.dim) || !int_at(jl, "mixer.vdim", D.vdim) || !int_at(jl, "mixer.conv", D.conv) ||
+                D.heads < 1 || D.kv_heads < 1 || D.heads % D.kv_heads || D.dim < 1 || D.vdim < 1 || D.conv < 1 || D.conv > 64) return bad("channel_delta needs positive 'heads', 'kv_heads' (a divisor of heads), 'dim', 'vdim' and 'conv' (1..64)");
+            if (D.dim > 1024) return bad("channel_delta key width above 1024");
+            if (!rank_of(p + "a1", D.decay_rank) || !rank_of(p + "g1", D.gate_rank)) return bad("tensors mix.a1 / mix.g1 [rank][width] are missing");
+            H.heads = D.heads; H.dim = D.dim; H.vdim = D.vdim;
+            H.state_index = n_state++;
+        } else if (type->str == "parallel") {
+            H.mixer = PI_MIXER_PARALLEL_SHIFT;
+            pi_gate_attention & A = H.left; pi_time_mix & R = H.shift;
+            if (!int_at(jl, "mixer.left.heads", A.heads) || !int_at(jl, "mixer.left.kv_heads", A.kv_heads) || !int_at(jl, "mixer.left.dim", A.dim) || !int_at(jl, "mixer.left.vdim", A.vdim) ||
+                A.heads < 1 || A.kv_heads < 1 || A.heads % A.kv_heads || A.dim < 1 || A.vdim < 1) return bad("mixer.left needs positive 'heads', 'kv_heads' (a divisor of heads), 'dim', 'vdim'");
+            if (!num_at(jl, "mixer.left.scale", d)) return bad("mixer.left needs 'scale'");
+            A.scale = (float) d; A.gated = false; A.weights = PI_WEIGHTS_SOFTMAX_SINK;
+            if (jl.at("mixer.left.softcap") && !jl.at("mixer.left.softcap")->is_null()) { if (!num_at(jl, "mixer.left.softcap", d) || d <= 0) return bad("mixer.left.softcap must be positive"); A.softcap = (float) d; }
+            if (jl.at("mixer.left.rot") && !jl.at("mixer.left.rot")->is_null()) {
+                if (!int_at(jl, "mixer.left.rot.dims", A.rot_dims) || !num_at(jl, "mixer.left.rot.base", d) || (A.rot_dims & 1) || A.rot_dims > A.dim) return bad("mixer.left.rot needs an even 'dims' <= dim and 'base'");
+                A.rot_base = (float) d;
+            }
+            if (jl.at("mixer.left.mask") && !jl.at("mixer.left.mask")->is_null() && (!int_at(jl, "mixer.left.mask.size", A.chunk) || A.chunk < 1)) return bad("mixer.left.mask needs a positive 'size'");
+            if (!int_at(jl, "mixer.right.heads", R.heads) || !int_at(jl, "mixer.right.dim", R.dim) || R.heads < 1 || R.dim < 1 || R.dim > 1024) return bad("mixer.right needs positive 'heads' and 'dim' (at most 1024)");
+            if (!rank_of(p + "right.w1", R.decay_rank)) return bad("tensor mix.right.w1 [rank][width] is missing");
+            R.width = hp.n_embd;
+            H.heads = A.heads; H.dim = A.dim; H.vdim = A.vdim;
+            H.cache_index = n_cache++; H.state_index = n_state++;
+        } else return bad("mixer type '" + type->str + "' is unknown (channel_delta, parallel)");
+        if (jl.has("mlp")) {
+            const json * kind = jl.at("mlp.kind");
+            if (!kind || !kind->is_str() || kind->str != "dense") return bad("feed-forward kind must be 'dense'");
+            if (!int_at(jl, "mlp.ff", H.ff) || H.ff < 1) return bad("a dense mlp needs 'ff'");
+            H.mlp = PI_MLP_DENSE_GEGLU; H.has_mlp = true;
+        }
+        hp.hybrid.push_back(std::move(H));
+    }
+    return true;
+}
+
 }  // namespace
 
 bool llama_model::ensure_loaded_hybrid(int n_positions, std::string & err) {
@@ -176,8 +259,9 @@ bool llama_model::ensure_loaded_hybrid(int n_positions, std::string & err) {
     }
     if (hp.own_head && !output) {
         if (!(output = L.matrix({ { "head", hp.n_vocab } }, width))) return false;
-        if (!(output_norm_b = L.vector("final.norm.b", width))) return false;
+        if (!hp.post_norm && !(output_norm_b = L.vector("final.norm.b", width))) return false;
     }
+    if (hp.pair_buckets > 0 && !pair_embd && !(pair_embd = L.matrix({ { "bigram", (int64_t) hp.pair_buckets + 1 } }, width))) return false;
     for (size_t i = 0; i < hp.hybrid.size(); i++) {
         const pi_hybrid_layer & H = hp.hybrid[i];
         pi_hybrid_weights & W = hweights[i];
@@ -188,6 +272,33 @@ bool llama_model::ensure_loaded_hybrid(int n_positions, std::string & err) {
         }
         if (H.weights != (int) i || W.loaded) continue;
         const std::string p = "l" + std::to_string(i) + ".";
+        if (hp.post_norm) {                                                // the norm after the sum: per sublayer a norm and a layer scale
+            if (!(W.norm1 = L.vector(p + "norm1", width)) || !(W.ls1 = L.vector(p + "ls1", width))) return false;
+            if (H.has_mlp && (!(W.norm2 = L.vector(p + "norm2", width)) || !(W.ls2 = L.vector(p + "ls2", width)))) return false;
+            if (H.mixer == PI_MIXER_CHANNEL_DELTA) {
+                const pi_channel_delta & D = H.delta;
+                const std::string m = p + "mix.";
+                const int64_t gd = (int64_t) D.kv_heads * D.dim, hd = (int64_t) D.heads * D.dim, hv = (int64_t) D.heads * D.vdim;
+                if (!(W.w_in = L.matrix({ { m + "q", gd }, { m + "k", gd }, { m + "v", hv }, { m + "a1", D.decay_rank }, { m + "g1", D.gate_rank }, { m + "b", D.heads } }, width))) return false;
+                if (!(W.w_a2 = L.matrix({ { m + "a2", hd } }, D.decay_rank)) || !(W.w_g2 = L.matrix({ { m + "g2", hv } }, D.gate_rank)) || !(W.w_o = L.matrix({ { m + "o", width } }, hv))) return false;
+                if (!(W.conv_w = L.vectors({ { m + "q.conv", gd }, { m + "k.conv", gd }, { m + "v.conv", hv } }, D.conv))) return false;
+                if (!(W.a_log = L.vector(m + "A_log", D.heads)) || !(W.dt_bias = L.vector(m + "dt_bias", hd)) || !(W.mix_norm = L.vector(m + "norm", D.vdim))) return false;
+            } else if (H.mixer == PI_MIXER_PARALLEL_SHIFT) {
+                const pi_gate_attention & A = H.left; const pi_time_mix & R = H.shift;
+                const std::string l = p + "mix.left.", r = p + "mix.right.";
+                if (!(W.w_in = L.matrix({ { l + "q", (int64_t) A.heads * A.dim }, { l + "k", (int64_t) A.kv_heads * A.dim }, { l + "v", (int64_t) A.kv_heads * A.vdim } }, width))) return false;
+                if (!(W.w_o = L.matrix({ { l + "o", width } }, (int64_t) A.heads * A.vdim)) || !(W.left_out = L.vector(l + "out", width))) return false;
+                if (!(W.rotary = pi_rotary_table_create(std::max(n_positions, 32), A.rot_dims, A.rot_base))) { err = std::string("rotation table: ") + pi_last_error(); return false; }
+                const int64_t inner = R.inner();
+                if (!(W.mu = L.vectors({ { r + "mu.r", width }, { r + "mu.k", width }, { r + "mu.v", width }, { r + "mu.g", width }, { r + "mu.w", width } }, 0))) return false;
+                if (!(W.w_r = L.matrix({ { r + "r", inner } }, width)) || !(W.w_k = L.matrix({ { r + "k", inner } }, width)) || !(W.w_v = L.matrix({ { r + "v", inner } }, width)) || !(W.w_g = L.matrix({ { r + "g", inner } }, width))) return false;
+                if (!(W.w_w1 = L.matrix({ { r + "w1", R.decay_rank } }, width)) || !(W.w_w2 = L.matrix({ { r + "w2", inner } }, R.decay_rank)) || !(W.w_o2 = L.matrix({ { r + "o", width } }, inner))) return false;
+                if (!(W.w0 = L.vector(r + "w0", inner)) || !(W.bonus = L.vector2(r + "u", R.heads, R.dim)) || !(W.mix_norm = L.vector(r + "norm", inner)) || !(W.right_out = L.vector(r + "out", width))) return false;
+            } else { err = "a block with the norm after the sum has no mixer of kind " + std::to_string((int) H.mixer); return false; }
+            if (H.mlp == PI_MLP_DENSE_GEGLU && (!(W.ff_up = L.matrix({ { p + "mlp.gate", H.ff }, { p + "mlp.up", H.ff } }, width)) || !(W.ff_down = L.matrix({ { p + "mlp.down", width } }, H.ff)))) return false;
+            W.loaded = true;
+            continue;
+        }
         if (H.mixer == PI_MIXER_PARALLEL) {
             const pi_gate_attention & A = H.left; const pi_ssd & R = H.right;
             const std::string l = p + "mix.left.", r = p + "mix.right.";
@@ -273,16 +384,17 @@ llama_model * load_hybrid_model(const std::string & folder, const llama_model_pa
     // the registry of folder-described architectures (GGUF files name theirs in general.architecture, model.cpp)
     if (arch->str == "Fasovik") hp.arch = PI_ARCH_FASOVIK;
     else if (arch->str == "Vikarax") hp.arch = PI_ARCH_VIKARAX;
-    else return fail("architecture '" + arch->str + "' is not one this engine builds (Fasovik, Vikarax)");
+    else if (arch->str == "Rafusun") hp.arch = PI_ARCH_RAFUSUN;
+    else return fail("architecture '" + arch->str + "' is not one this engine builds (Fasovik, Vikarax, Rafusun)");
     m->name = arch->str;
     double d;
     if (!int_at(cfg, "vocab", hp.n_vocab) || !int_at(cfg, "width", hp.n_embd) || hp.n_vocab < 1 || hp.n_embd < 1) return fail("'vocab' and 'width' must be positive integers");
-    if (hp.arch == PI_ARCH_VIKARAX) {
+    if (hp.arch == PI_ARCH_VIKARAX || hp.arch == PI_ARCH_RAFUSUN) {
         std::string what;
-        if (!read_vikarax_config(cfg, hp, what)) return fail(what);
+        if (!params.vocab_only && !m->st_file.open(folder + "/model.safetensors", err)) { fprintf(stderr, "llama_load_model_from_file: %s\n", err.c_str()); return nullptr; }
+        if (hp.arch == PI_ARCH_VIKARAX ? !read_vikarax_config(cfg, hp, what) : !read_rafusun_config(cfg, params.vocab_only ? nullptr : &m->st_file, hp, what)) return fail(what);
         m->hweights.resize((size_t) hp.n_layer);
         if (!params.vocab_only) {
-            if (!m->st_file.open(folder + "/model.safetensors", err)) { fprintf(stderr, "llama_load_model_from_file: %s\n", err.c_str()); return nullptr; }
             for (const auto & kv : m->st_file.tensors) { m->n_elements += (uint64_t) kv.second.elements(); m->n_bytes += kv.second.nbytes; }
             const st_tensor * e = m->st_file.tensor("embed"), * h = m->st_file.tensor("head");
             if (!e || e->shape != std::vector<int64_t>{ hp.n_vocab, hp.n_embd } || !h || h->shape != e->shape) return fail("tensors 'embed' and 'head' are missing or not [vocab][width]");

@@ -11,7 +11,7 @@ namespace pi {
 
 class state_slots {
 public:
-    explicit state_slots(int n_slots) : owner_(n_slots, -1), fresh_(n_slots, 0) {}
+    explicit state_slots(int n_slots) : owner_(n_slots, -1), fresh_(n_slots, 0), last_(n_slots, -1) {}
     int  size() const { return (int) owner_.size(); }
     int  used() const { int n = 0; for (int o : owner_) n += o >= 0; return n; }
     int  find(int seq) const { for (int i = 0; i < size(); i++) if (owner_[i] == seq) return i; return -1; }
@@ -19,7 +19,7 @@ public:
     int  acquire(int seq) {
         int s = find(seq);
         if (s >= 0) return s;
-        for (int i = 0; i < size(); i++) if (owner_[i] < 0) { owner_[i] = seq; fresh_[i] = 1; return i; }
+        for (int i = 0; i < size(); i++) if (owner_[i] < 0) { owner_[i] = seq; fresh_[i] = 1; last_[i] = -1; return i; }
         return -1;
     }
     // true once per allotment: the caller's next run must start the slot's state from zero
@@ -30,9 +30,13 @@ public:
     void keep(int seq) { for (int i = 0; i < size(); i++) if (owner_[i] != seq) { owner_[i] = -1; fresh_[i] = 0; } }
     void clear() { for (int i = 0; i < size(); i++) { owner_[i] = -1; fresh_[i] = 0; } }
     int  owner(int slot) const { return owner_[slot]; }
+    // the last token the slot's sequence was fed (-1: none yet): models whose embedding looks at the previous token
+    int  last_token(int slot) const { return last_[slot]; }
+    void set_last_token(int slot, int token) { last_[slot] = token; }
 private:
     std::vector<int32_t> owner_;
     std::vector<uint8_t> fresh_;
+    std::vector<int32_t> last_;
 };
 
 }  // namespace pi

@@ -1,0 +1,341 @@
+// Operators of blocks whose norm comes AFTER the sum (x <- R(alpha x + ls * sublayer(x)) * w) and of recurrent mixers whose state decays per key channel:
+//
+//   k_embed_pair         token row * scale + a row of a second table (a hashed pair embedding: the host names the row of every token)
+//   k_rms_post           the end of a sublayer in one launch: [the mean of two RMS-normed branch outputs ->] layer scale -> + alpha x -> RMS norm [-> a second RMS norm for what reads x next]
+//   k_token_shift(_walk) m_s = h + (h_prev - h) * mu_s for several s at once; h_prev of a sequence's first token of the pass comes from (and its last token goes to) the sequence's state
+//   k_channel_recurrence per head a [dim][vdim] state, per token and key channel a decay.  Two rules:
+//                          delta   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q        (the read-out sees the token's own write)
+//                          bonus   o = (S + diag(b) k v^T)^T q;  S <- diag(g) S + k v^T                         (the read-out sees the token through the bonus only)
+//                        decays arrive raw and are formed here (exp(-exp(raw + bias)) or exp(-exp(A_h) softplus(raw + bias))), q / k can be made unit vectors here, beta is sigmoid(raw)
+//   k_head_norm_gate     every head's output divided by its root mean square, * weight (shared by the heads or one per head), * gate (as is, sigmoid or silu of it)
+//
+// Everything is fp32 in both precisions of the engine.
+#include "ops_common.h"
+#include "kernel_timing.h"
+
+#include <algorithm>
+#include <cmath>
+
+#define CM_FRESH (1 << 30)
+
+static __device__ __forceinline__ float cm_widen(uint16_t b) { return __uint_as_float((uint32_t) b << 16); }
+static __device__ __forceinline__ float cm_sigmoid(float v) { return 1.0f / (1.0f + expf(-v)); }
+static __device__ __forceinline__ float cm_softplus(float z) { return z > 20.0f ? z : log1pf(expf(z)); }        // (beyond 20 the two agree to the last bit of fp32)
+static __device__ __forceinline__ float cm_block_sum(float v, float * red) {          // sum over the block's threads (every thread gets it); red: 4 floats, reusable after the call
+    v = pi_lanes_sum<64>(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float s = 0.0f;
+    for (int i = 0; i < (int) (blockDim.x >> 6); i++) s += red[i];
+    return s;
+}
+
+// ---- embedding: token row * scale + a row of a second table ---------------------------------------------------------------------------------------------
+__global__ void k_embed_pair(const uint16_t * __restrict__ table, int64_t width, int64_t n_rows, const int32_t * __restrict__ tokens, float scale, const uint16_t * __restrict__ table2, int64_t n_rows2,
+                             const int32_t * __restrict__ rows2, float * __restrict__ out, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.x;
+    const int64_t row = tokens[t], row2 = rows2[t];
+    const bool ok = row >= 0 && row < n_rows, ok2 = row2 >= 0 && row2 < n_rows2;
+    for (int64_t i = threadIdx.x; i < width; i += blockDim.x)
+        out[(int64_t) t * width + i] = (ok ? cm_widen(table[row * width + i]) * scale : 0.0f) + (ok2 ? cm_widen(table2[row2 * width + i]) : 0.0f);
+}
+extern "C" int pi_op_embed_pair(const pi_weight * w, const int32_t * tokens, int n_tok, float scale, const pi_weight * w2, const int32_t * rows2, float * out, void * stream) {
+    if (!w || w->type != PI_BF16 || !w2 || w2->type != PI_BF16 || w->ne0 != w2->ne0) { pi_set_error("pi_op_embed_pair: two bfloat16 tables of the same width are required"); return -1; }
+    if (n_tok <= 0) return 0;
+    PI_KT_LAUNCH(PI_KT_OTHER, PI_BF16, 1, 8.0 * w->ne0 * n_tok, k_embed_pair, dim3((unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, (const uint16_t *) w->p0, w->ne0, w->ne1, tokens, scale,
+                 (const uint16_t *) w2->p0, w2->ne1, rows2, out, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+
+// ---- the end of a sublayer whose norm comes after the sum ------------------------------------------------------------------------------------------------
+// per token row:  m = b ? mb * (R(a) * wa + R(b) * wb) : a;   v = alpha * x + ls * m;   out = R(v) * w;   (w_next)  out_next = R(out) * w_next.   R(y) = y / sqrt(mean(y^2) + eps).
+// A thread keeps its NPT values of every row in registers; out may be x.
+template <int NPT>
+__global__ void __launch_bounds__(256) k_rms_post(const float * __restrict__ a, int64_t as, const float * __restrict__ wa, const float * __restrict__ b, int64_t bs, const float * __restrict__ wb, float mb,
+                                                  const float * __restrict__ ls, const float * __restrict__ x, int64_t xs, float alpha, const float * __restrict__ w, float eps, int n,
+                                                  float * __restrict__ out, int64_t os, const float * __restrict__ w_next, float * __restrict__ out_next, int64_t ons, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    __shared__ float red[4];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    float m[NPT], v[NPT];
+#pragma unroll
+    for (int j = 0; j < NPT; j++) { const int i = j * 256 + tid; m[j] = i < n ? a[(int64_t) t * as + i] : 0.0f; }
+    if (b) {
+        float sa = 0.0f, sb = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NPT; j++) { const int i = j * 256 + tid; v[j] = i < n ? b[(int64_t) t * bs + i] : 0.0f; sa = fmaf(m[j], m[j], sa); sb = fmaf(v[j], v[j], sb); }
+        sa = cm_block_sum(sa, red); sb = cm_block_sum(sb, red);
+        const float ia = 1.0f / sqrtf(sa / (float) n + eps), ib = 1.0f / sqrtf(sb / (float) n + eps);
+#pragma unroll
+        for (int j = 0; j < NPT; j++) { const int i = j * 256 + tid; if (i < n) m[j] = mb * (m[j] * ia * wa[i] + v[j] * ib * wb[i]); }
+    }
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NPT; j++) {
+        const int i = j * 256 + tid;
+        v[j] = i < n ? fmaf(alpha, x[(int64_t) t * xs + i], (ls ? ls[i] : 1.0f) * m[j]) : 0.0f;
+        ss = fmaf(v[j], v[j], ss);
+    }
+    ss = cm_block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float) n + eps);
+    float s2 = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NPT; j++) { const int i = j * 256 + tid; if (i < n) { v[j] = v[j] * inv * w[i]; out[(int64_t) t * os + i] = v[j]; s2 = fmaf(v[j], v[j], s2); } }
+    if (!w_next) return;
+    s2 = cm_block_sum(s2, red);
+    const float inv2 = 1.0f / sqrtf(s2 / (float) n + eps);
+#pragma unroll
+    for (int j = 0; j < NPT; j++) { const int i = j * 256 + tid; if (i < n) out_next[(int64_t) t * ons + i] = v[j] * inv2 * w_next[i]; }
+}
+extern "C" int pi_op_rms_post(const float * a, int64_t a_stride, const float * wa, const float * b, int64_t b_stride, const float * wb, float mean_mult, const float * layer_scale, const float * x, int64_t x_stride,
+                              float alpha, const float * w, float eps, int n, int n_tok, float * out, int64_t out_stride, const float * w_next, float * out_next, int64_t out_next_stride, void * stream) {
+    if (n_tok <= 0 || n <= 0) return 0;
+    if (n > 256 * 32) { pi_set_error("pi_op_rms_post: rows of %d values (at most %d)", n, 256 * 32); return -1; }
+    if (b && (!wa || !wb)) { pi_set_error("pi_op_rms_post: two inputs need the weights of their norms"); return -1; }
+    if (w_next && !out_next) { pi_set_error("pi_op_rms_post: a second norm needs a place for its result"); return -1; }
+    const double bytes = 4.0 * n * n_tok * (3.0 + (b ? 1 : 0) + (w_next ? 1 : 0));
+#define RP_GO(N) PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, bytes, k_rms_post<N>, dim3((unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, a, a_stride, wa, b, b_stride, wb, mean_mult, layer_scale, x, x_stride, alpha, w, eps, n, \
+                              out, out_stride, w_next, out_next, out_next_stride, pi_abort_word())
+    if (n <= 256 * 2) RP_GO(2); else if (n <= 256 * 4) RP_GO(4); else if (n <= 256 * 8) RP_GO(8); else if (n <= 256 * 16) RP_GO(16); else RP_GO(32);
+#undef RP_GO
+    PI_CHECK_LAUNCH(); return 0;
+}
+
+// ---- token shift: every mix of a token with the token before it ------------------------------------------------------------------------------------------------
+// out[t][s][i] = h[t][i] + (prev[i] - h[t][i]) * mu[s][i], s < n_mix; prev = h[t - 1] inside a sequence's run, the sequence's state (zeros on a fresh slot) at the run's first token.
+// rec as for the recurrences; state: [slots][n].  grid (token, blocks of 256 values)
+__global__ void __launch_bounds__(256) k_token_shift(const float * __restrict__ h, int64_t hs, int n, const float * __restrict__ mu, int n_mix, const float * __restrict__ state, const int32_t * __restrict__ rec,
+                                                     float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.x, i = blockIdx.y * 256 + threadIdx.x;
+    if (i >= n) return;
+    const int word = rec[t], slot = word & ~CM_FRESH;
+    const bool inside = t > 0 && (rec[t - 1] & ~CM_FRESH) == slot;
+    const float cur = h[(int64_t) t * hs + i];
+    const float prev = inside ? h[(int64_t) (t - 1) * hs + i] : (word & CM_FRESH) ? 0.0f : state[(int64_t) slot * n + i];
+    const float d = prev - cur;
+    for (int s = 0; s < n_mix; s++) out[(int64_t) t * os + (int64_t) s * n + i] = fmaf(d, mu[(int64_t) s * n + i], cur);
+}
+// a run's last token becomes the sequence's state (its own launch: the run's first token reads the state in the launch above)
+__global__ void __launch_bounds__(256) k_token_shift_state(const float * __restrict__ h, int64_t hs, int n, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.x, i = blockIdx.y * 256 + threadIdx.x;
+    const int slot = rec[t] & ~CM_FRESH;
+    if (i >= n || (t + 1 < n_tok && (rec[t + 1] & ~CM_FRESH) == slot)) return;
+    state[(int64_t) slot * n + i] = h[(int64_t) t * hs + i];
+}
+// short passes in ONE launch: the thread of a run's first token walks the run for its value and leaves the state, so nothing it writes is read by another thread
+__global__ void __launch_bounds__(256) k_token_shift_walk(const float * __restrict__ h, int64_t hs, int n, const float * __restrict__ mu, int n_mix, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok,
+                                                          float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.x, i = blockIdx.y * 256 + threadIdx.x;
+    const int word = rec[t], slot = word & ~CM_FRESH;
+    if (i >= n || (t > 0 && (rec[t - 1] & ~CM_FRESH) == slot)) return;
+    float prev = (word & CM_FRESH) ? 0.0f : state[(int64_t) slot * n + i];
+    for (int tt = t; tt < n_tok && (rec[tt] & ~CM_FRESH) == slot; tt++) {
+        const float cur = h[(int64_t) tt * hs + i], d = prev - cur;
+        for (int s = 0; s < n_mix; s++) out[(int64_t) tt * os + (int64_t) s * n + i] = fmaf(d, mu[(int64_t) s * n + i], cur);
+        prev = cur;
+    }
+    state[(int64_t) slot * n + i] = prev;
+}
+#define TS_WALK_MAX_TOKENS 32
+extern "C" int pi_op_token_shift(const float * h, int64_t h_stride, int n, const float * mu_dev, int n_mix, float * state_dev, const int32_t * rec_dev, int n_tok, float * out, int64_t out_stride, void * stream) {
+    if (n_tok <= 0 || n <= 0) return 0;
+    if (n_mix < 1 || out_stride < (int64_t) n_mix * n) { pi_set_error("pi_op_token_shift: %d mixes of %d values do not fit rows %lld floats apart", n_mix, n, (long long) out_stride); return -1; }
+    if (out == h) { pi_set_error("pi_op_token_shift: the output may not overwrite the input (the next token reads it)"); return -1; }
+    hipStream_t s = (hipStream_t) stream;
+    const dim3 grid((unsigned) n_tok, (unsigned) ((n + 255) / 256));
+    const double bytes = 4.0 * n * n_tok * (1.0 + n_mix) + 4.0 * n * n_mix;
+    if (n_tok <= TS_WALK_MAX_TOKENS) {
+        PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, bytes, k_token_shift_walk, grid, dim3(256), 0, s, h, h_stride, n, mu_dev, n_mix, state_dev, rec_dev, n_tok, out, out_stride, pi_abort_word());
+        PI_CHECK_LAUNCH(); return 0;
+    }
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, bytes, k_token_shift, grid, dim3(256), 0, s, h, h_stride, n, mu_dev, n_mix, state_dev, rec_dev, out, out_stride, pi_abort_word());
+    PI_CHECK_LAUNCH();
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 8.0 * n, k_token_shift_state, grid, dim3(256), 0, s, h, h_stride, n, state_dev, rec_dev, n_tok, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+
+// ---- recurrences with a decay per key channel ------------------------------------------------------------------------------------------------------------------
+// Workgroup (head, block of value columns, run of the pass): thread (column j, part sp of R) keeps S[i][j] for its DPT rows i in registers and walks the run's tokens in order; q, k,
+// the decays and v of CR_TB tokens at a time are staged (and finished: decays formed, unit vectors, sigmoid) in LDS.  A value column never meets another: o_j, u_j and S[:, j]
+// depend on column j alone, so the only exchange is the sum over the R parts of a column (neighbouring lanes).
+//   delta:  S <- g S;  a = S^T k, c = S^T q (one pass over the registers);  u = beta (v - a);  o = c + u (k . q);  S <- S + k u
+//   bonus:  c = S^T q;  o = c + v (sum_i q_i b_i k_i);  S <- g S + k v
+#define CR_TB 32
+#define CR_MAXRUNS 256
+template <int DPT, int RULE>
+__global__ void __launch_bounds__(256) k_channel_recurrence(const float * __restrict__ q, int64_t qs, const float * __restrict__ k, int64_t ks, const float * __restrict__ v, int64_t vs,
+                                                            const float * __restrict__ draw, int64_t ds, int decay_mode, const float * __restrict__ dbias, const float * __restrict__ a_log,
+                                                            const float * __restrict__ braw, int64_t bs, const float * __restrict__ bonus, int qk_unit, float q_mult,
+                                                            int heads, int hpg, int dim, int vdim, int R, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok,
+                                                            float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    extern __shared__ float lds[];                // q [CR_TB][dim] | k [CR_TB][dim] | g [CR_TB][dim] | v [CR_TB][cols]
+    __shared__ int seg[4], bnd[CR_MAXRUNS], nbnd; // first token, length, slot word of this workgroup's run, first token of the next run
+    __shared__ float beta_t[CR_TB], dot_t[CR_TB];
+    const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
+    // run number blockIdx.z of the pass (a run: the consecutive tokens of one slot).  Every thread looks at its own tokens for a run's first one, the few found are ranked by position
+    if (tid == 0) { nbnd = 0; seg[0] = 0; seg[1] = 0; seg[2] = -1; seg[3] = n_tok; }
+    __syncthreads();
+    for (int t = tid; t < n_tok; t += blockDim.x)
+        if (t == 0 || (rec[t] & ~CM_FRESH) != (rec[t - 1] & ~CM_FRESH)) { const int at = atomicAdd(&nbnd, 1); if (at < CR_MAXRUNS) bnd[at] = t; }
+    __syncthreads();
+    const int n_runs = min(nbnd, CR_MAXRUNS);
+    for (int i = tid; i < n_runs; i += blockDim.x) {
+        int rank = 0;
+        for (int o = 0; o < n_runs; o++) rank += bnd[o] < bnd[i];
+        if (rank == (int) blockIdx.z) { seg[0] = bnd[i]; seg[2] = rec[bnd[i]]; }
+        if (rank == (int) blockIdx.z + 1) seg[3] = bnd[i];
+    }
+    __syncthreads();
+    if (tid == 0 && seg[2] >= 0) seg[1] = seg[3] - seg[0];
+    __syncthreads();
+    const int first = seg[0], len = seg[1], word = seg[2];
+    if (len == 0 || word < 0) return;
+    const int slot = word & ~CM_FRESH;
+    const int cols = blockDim.x / R;
+    const int j = blockIdx.y * cols + tid / R, sp = tid % R;
+    const bool col_ok = j < vdim;
+    const int hq = h / hpg;                                            // the q / k head this head reads
+    float * S_hbm = state + ((int64_t) slot * heads + h) * dim * vdim;
+    float S[DPT];
+#pragma unroll
+    for (int ii = 0; ii < DPT; ii++) {
+        const int i = sp * DPT + ii;
+        S[ii] = (col_ok && i < dim && !(word & CM_FRESH)) ? S_hbm[(int64_t) i * vdim + j] : 0.0f;
+    }
+    float * qt = lds, * kt = qt + CR_TB * dim, * gt = kt + CR_TB * dim, * vt = gt + CR_TB * dim;
+    const float ah = decay_mode == 2 ? expf(a_log[h]) : 0.0f;
+    for (int t0 = 0; t0 < len; t0 += CR_TB) {
+        const int nt = min(CR_TB, len - t0);
+        __syncthreads();
+        for (int idx = tid; idx < nt * dim; idx += blockDim.x) {
+            const int tt = idx / dim, i = idx % dim;
+            const int64_t tok = first + t0 + tt;
+            qt[idx] = q[tok * qs + (int64_t) hq * dim + i];
+            kt[idx] = k[tok * ks + (int64_t) hq * dim + i];
+            float d = draw[tok * ds + (int64_t) h * dim + i];
+            if (decay_mode == 1) d = expf(-expf(d + (dbias ? dbias[h * dim + i] : 0.0f)));
+            else if (decay_mode == 2) d = expf(-ah * cm_softplus(d + (dbias ? dbias[h * dim + i] : 0.0f)));
+            gt[idx] = d;
+        }
+        if (tid < nt) beta_t[tid] = braw ? cm_sigmoid(braw[(int64_t) (first + t0 + tid) * bs + h]) : 1.0f;
+        for (int idx = tid; idx < nt * cols; idx += blockDim.x) {
+            const int tt = idx / cols, jj = blockIdx.y * cols + idx % cols;
+            vt[idx] = jj < vdim ? v[(int64_t) (first + t0 + tt) * vs + (int64_t) h * vdim + jj] : 0.0f;
+        }
+        __syncthreads();
+        for (int tt = wave; tt < nt; tt += nw) {                          // a wave per token: unit vectors, then the token's scalar (k . q, or sum q b k)
+            float * qr = qt + tt * dim, * kr = kt + tt * dim;
+            if (qk_unit) {
+                float sq = 0.0f, sk = 0.0f;
+                for (int i = lane; i < dim; i += 64) { sq = fmaf(qr[i], qr[i], sq); sk = fmaf(kr[i], kr[i], sk); }
+                const float iq = q_mult / sqrtf(pi_lanes_sum<64>(sq) + 1e-6f), ik = 1.0f / sqrtf(pi_lanes_sum<64>(sk) + 1e-6f);
+                for (int i = lane; i < dim; i += 64) { qr[i] *= iq; kr[i] *= ik; }
+            } else if (q_mult != 1.0f) for (int i = lane; i < dim; i += 64) qr[i] *= q_mult;
+            float d = 0.0f;
+            for (int i = lane; i < dim; i += 64) d = fmaf(RULE == 1 && bonus ? qr[i] * bonus[h * dim + i] : qr[i], kr[i], d);      // (a lane re-reads only what it wrote itself)
+            d = pi_lanes_sum<64>(d);
+            if (lane == 0) dot_t[tt] = d;
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nt; tt++) {
+            const float vj = vt[tt * cols + tid / R];
+            const float * kr = kt + tt * dim + sp * DPT, * qr = qt + tt * dim + sp * DPT, * gr = gt + tt * dim + sp * DPT;
+            float a = 0.0f, c = 0.0f, o;
+            if (RULE == 0) {
+#pragma unroll
+                for (int ii = 0; ii < DPT; ii++)
+                    if (sp * DPT + ii < dim) { S[ii] *= gr[ii]; a = fmaf(S[ii], kr[ii], a); c = fmaf(S[ii], qr[ii], c); }
+            } else {
+#pragma unroll
+                for (int ii = 0; ii < DPT; ii++)
+                    if (sp * DPT + ii < dim) c = fmaf(S[ii], qr[ii], c);
+            }
+            if (R == 2) { if (RULE == 0) a += pi_partner<1>(a); c += pi_partner<1>(c); }
+            else if (R == 4) { if (RULE == 0) { a += pi_partner<2>(a); a += pi_partner<1>(a); } c += pi_partner<2>(c); c += pi_partner<1>(c); }
+            else for (int d = R >> 1; d > 0; d >>= 1) { if (RULE == 0) a += __shfl_xor(a, d, PI_WAVE); c += __shfl_xor(c, d, PI_WAVE); }
+            if (RULE == 0) {
+                const float u = beta_t[tt] * (vj - a);
+                o = fmaf(u, dot_t[tt], c);
+#pragma unroll
+                for (int ii = 0; ii < DPT; ii++) if (sp * DPT + ii < dim) S[ii] = fmaf(kr[ii], u, S[ii]);
+            } else {
+                o = fmaf(vj, dot_t[tt], c);
+#pragma unroll
+                for (int ii = 0; ii < DPT; ii++) if (sp * DPT + ii < dim) S[ii] = fmaf(kr[ii], vj, gr[ii] * S[ii]);
+            }
+            if (col_ok && sp == 0) out[(int64_t) (first + t0 + tt) * os + (int64_t) h * vdim + j] = o;
+        }
+    }
+    if (col_ok)
+#pragma unroll
+        for (int ii = 0; ii < DPT; ii++) { const int i = sp * DPT + ii; if (i < dim) S_hbm[(int64_t) i * vdim + j] = S[ii]; }
+}
+
+#define CR_LDS_MAX (150 * 1024)
+template <int DPT, int RULE> static int cr_reserve_one() { PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_channel_recurrence<DPT, RULE>, hipFuncAttributeMaxDynamicSharedMemorySize, CR_LDS_MAX)); return 0; }
+extern "C" int pi_op_channel_recurrence_reserve(void) {
+    static bool done = false;
+    if (done) return 0;
+    if (cr_reserve_one<8, 0>() || cr_reserve_one<16, 0>() || cr_reserve_one<32, 0>() || cr_reserve_one<8, 1>() || cr_reserve_one<16, 1>() || cr_reserve_one<32, 1>()) return -1;
+    done = true;
+    return 0;
+}
+extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_stride, const float * k, int64_t k_stride, const float * v, int64_t v_stride, const float * decay_raw, int64_t decay_stride, int decay_mode,
+                                        const float * decay_bias_dev, const float * a_log_dev, const float * beta_raw, int64_t beta_stride, const float * bonus_dev, int qk_unit, float q_mult,
+                                        int heads, int qk_heads, int dim, int vdim, float * state_dev, const int32_t * rec_dev, int n_tok, int max_segments, float * out, int64_t out_stride, void * stream) {
+    if (n_tok <= 0) return 0;
+    if (rule != PI_RULE_DELTA && rule != PI_RULE_BONUS) { pi_set_error("pi_op_channel_recurrence: rule %d is unknown", rule); return -1; }
+    if (qk_heads < 1 || heads % qk_heads) { pi_set_error("pi_op_channel_recurrence: %d heads do not divide over %d query / key heads", heads, qk_heads); return -1; }
+    if (dim <= 0 || vdim <= 0 || heads <= 0 || dim > 1024) { pi_set_error("pi_op_channel_recurrence: head sizes %d x %d outside the kernel's range (key width <= 1024)", dim, vdim); return -1; }
+    if (decay_mode < 0 || decay_mode > 2 || (decay_mode == 2 && !a_log_dev) || !decay_raw) { pi_set_error("pi_op_channel_recurrence: decays (mode %d) are missing a part", decay_mode); return -1; }
+    if (max_segments > CR_MAXRUNS) { pi_set_error("pi_op_channel_recurrence: at most %d sequences in a pass", CR_MAXRUNS); return -1; }
+    const int dpt = dim <= 8 ? 8 : dim <= 16 ? 16 : 32;                // state values a thread keeps in registers
+    int R = 1; while (R * dpt < dim) R *= 2;
+    const int threads = std::min(256, (vdim * R + 63) / 64 * 64);
+    const int cols = threads / R;
+    const dim3 grid((unsigned) heads, (unsigned) ((vdim + cols - 1) / cols), (unsigned) std::max(1, std::min(n_tok, max_segments)));
+    const size_t lds = ((size_t) 3 * CR_TB * dim + (size_t) CR_TB * cols) * sizeof(float);
+    if (lds > CR_LDS_MAX) { pi_set_error("pi_op_channel_recurrence: a key width of %d needs %zu bytes of LDS (at most %d)", dim, lds, CR_LDS_MAX); return -1; }
+    if (lds > 48 * 1024 && pi_op_channel_recurrence_reserve() != 0) return -1;
+    const double bytes = 4.0 * n_tok * heads * (3.0 * dim + 2.0 * vdim) + 8.0 * heads * dim * vdim;
+    hipStream_t s = (hipStream_t) stream;
+    const int nta = std::min(n_tok, PI_KT_MAXNT - 1);
+#define CR_GO(D, RL) PI_KT_LAUNCH(PI_KT_ATT, 0, nta, bytes, (k_channel_recurrence<D, RL>), grid, dim3(threads), lds, s, q, q_stride, k, k_stride, v, v_stride, decay_raw, decay_stride, decay_mode, decay_bias_dev, a_log_dev, \
+                                  beta_raw, beta_stride, bonus_dev, qk_unit, q_mult, heads, heads / qk_heads, dim, vdim, R, state_dev, rec_dev, n_tok, out, out_stride, pi_abort_word())
+    if (rule == PI_RULE_DELTA) { if (dpt == 8) CR_GO(8, 0); else if (dpt == 16) CR_GO(16, 0); else CR_GO(32, 0); }
+    else                       { if (dpt == 8) CR_GO(8, 1); else if (dpt == 16) CR_GO(16, 1); else CR_GO(32, 1); }
+#undef CR_GO
+    PI_CHECK_LAUNCH(); return 0;
+}
+
+// ---- per-head RMS norm, weight, gate ------------------------------------------------------------------------------------------------------------------------------
+// out[t][h][i] = y[t][h][i] / sqrt(mean_i(y[t][h]^2) + eps) * w[(w_per_head ? h * n : 0) + i] * act(gate[t][h][i]);  a wave per (token, head); out may be y
+__global__ void __launch_bounds__(256) k_head_norm_gate(const float * __restrict__ y, int64_t ys, int heads, int n, const float * __restrict__ w, int w_per_head, const float * __restrict__ gate, int64_t gs, int gate_act,
+                                                        float eps, float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.x, h = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (h >= heads) return;
+    const float * yr = y + (int64_t) t * ys + (int64_t) h * n;
+    float ss = 0.0f;
+    for (int i = lane; i < n; i += 64) ss = fmaf(yr[i], yr[i], ss);
+    const float inv = 1.0f / sqrtf(pi_lanes_sum<64>(ss) / (float) n + eps);
+    for (int i = lane; i < n; i += 64) {
+        float g = gate ? gate[(int64_t) t * gs + (int64_t) h * n + i] : 1.0f;
+        if (gate && gate_act == PI_ACT_SIGMOID) g = cm_sigmoid(g);
+        else if (gate && gate_act == PI_ACT_SILU) g = g / (1.0f + expf(-g));
+        out[(int64_t) t * os + (int64_t) h * n + i] = yr[i] * inv * w[(w_per_head ? h * n : 0) + i] * g;
+    }
+}
+extern "C" int pi_op_head_norm_gate(const float * y, int64_t y_stride, int heads, int n, const float * w_dev, int w_per_head, const float * gate, int64_t gate_stride, int gate_act, float eps, int n_tok,
+                                    float * out, int64_t out_stride, void * stream) {
+    if (n_tok <= 0 || heads <= 0 || n <= 0) return 0;
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 12.0 * n_tok * heads * n, k_head_norm_gate, dim3((unsigned) n_tok, (unsigned) ((heads + 3) / 4)), dim3(256), 0, (hipStream_t) stream, y, y_stride, heads, n, w_dev, w_per_head,
+                 gate, gate_stride, gate_act, eps, out, out_stride, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}

@@ -30,6 +30,8 @@ static __device__ __forceinline__ float dn_act(float v, int act) {
         case PI_ACT_SILU:     return v / (1.0f + expf(-v));
         case PI_ACT_SIGMOID:  return 1.0f / (1.0f + expf(-v));
         case PI_ACT_RELU_SQR: { const float r = fmaxf(v, 0.0f); return r * r; }
+        case PI_ACT_TANH:     return tanhf(v);
+        case PI_ACT_GELU_TANH: return 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
         default:              return v;
     }
 }

@@ -103,6 +103,75 @@ extern "C" int pi_op_qkv_prepare(const float * q, const float * k, const float *
     PI_CHECK_LAUNCH(); return 0;
 }
 
+// the same with the order and the pairing as parameters.  norm_first: R(.) * w, then the rotation (as above), else the rotation first and R(.) * w over the rotated head; w may be absent (1);
+// pairing PI_PAIR_HALVES: dimension i with i + dims / 2, PI_PAIR_NEIGHBOURS: 2i with 2i + 1 (angle number i either way); v_norm = 0: value heads go to their cell as they are
+__global__ void __launch_bounds__(64) k_qkv_prepare_any(const float * __restrict__ q, const float * __restrict__ k, const float * __restrict__ v, int64_t stride, const float * __restrict__ qw,
+                                                        const float * __restrict__ kw, float eps, int H, int G, int D, int V, const float2 * __restrict__ rot, int half, int n_pos, int norm_first, int pairing, int v_norm,
+                                                        const int32_t * __restrict__ pos, float * __restrict__ q_out, int64_t qos, float * __restrict__ kc, float * __restrict__ vc,
+                                                        int32_t * __restrict__ cell_pos, const int32_t * __restrict__ dyn, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.x, slot = blockIdx.y, lane = threadIdx.x;
+    const int cell = pi_cell_of(dyn, 0, t);
+    const int p = pos[t];
+    if (slot == 0 && lane == 0) cell_pos[cell] = p;
+    if (slot >= H + G) {
+        const int g = slot - H - G;
+        const float * src = v + (int64_t) t * stride + (int64_t) g * V;
+        float inv = 1.0f;
+        if (v_norm) {
+            float ss = 0.0f;
+            for (int i = lane; i < V; i += 64) ss = fmaf(src[i], src[i], ss);
+            inv = 1.0f / sqrtf(pi_lanes_sum<64>(ss) / (float) V + eps);
+        }
+        float * dst = vc + ((int64_t) cell * G + g) * V;
+        for (int i = lane; i < V; i += 64) dst[i] = v_norm ? src[i] * inv : src[i];
+        return;
+    }
+    const bool is_q = slot < H;
+    const int h = is_q ? slot : slot - H;
+    const float * src = (is_q ? q : k) + (int64_t) t * stride + (int64_t) h * D;
+    const float * w = is_q ? qw : kw;
+    float * dst = is_q ? q_out + (int64_t) t * qos + (int64_t) h * D : kc + ((int64_t) cell * G + h) * D;
+    float inv1 = 1.0f;
+    if (norm_first) {
+        float ss = 0.0f;
+        for (int i = lane; i < D; i += 64) ss = fmaf(src[i], src[i], ss);
+        inv1 = 1.0f / sqrtf(pi_lanes_sum<64>(ss) / (float) D + eps);
+    }
+    const float2 * cs = rot + (int64_t) min(p, n_pos - 1) * half;
+    auto before = [&](int i) { return norm_first ? src[i] * inv1 * (w ? w[i] : 1.0f) : src[i]; };
+    auto turned = [&](int i) {
+        float y = before(i);
+        if (i < 2 * half) {
+            const bool lead = pairing == PI_PAIR_NEIGHBOURS ? !(i & 1) : i < half;                       // the pair's first member: u cos - v sin; its second: v cos + u sin
+            const int j = pairing == PI_PAIR_NEIGHBOURS ? (i ^ 1) : (i < half ? i + half : i - half), f = pairing == PI_PAIR_NEIGHBOURS ? (i >> 1) : (i < half ? i : i - half);
+            const float o = before(j);
+            const float2 c = cs[f];
+            y = lead ? y * c.x - o * c.y : y * c.x + o * c.y;
+        }
+        return y;
+    };
+    if (norm_first) { for (int i = lane; i < D; i += 64) dst[i] = turned(i); return; }
+    float ss = 0.0f;
+    for (int i = lane; i < D; i += 64) { const float y = turned(i); ss = fmaf(y, y, ss); }
+    const float inv = 1.0f / sqrtf(pi_lanes_sum<64>(ss) / (float) D + eps);
+    for (int i = lane; i < D; i += 64) dst[i] = turned(i) * inv * (w ? w[i] : 1.0f);
+}
+extern "C" int pi_op_qkv_prepare_ex(const float * q, const float * k, const float * v, int64_t stride, const float * q_norm_w, const float * k_norm_w, float eps, int heads, int kv_heads, int dim, int vdim,
+                                    const void * rotary_table, int norm_first, int pairing, int v_norm, const int32_t * pos_dev, int n_tok, float * q_out, int64_t q_out_stride, float * k_cache, float * v_cache,
+                                    int32_t * cell_pos_dev, const int32_t * dyn_dev, void * stream) {
+    if (n_tok <= 0) return 0;
+    const pi_rotary_table * rt = (const pi_rotary_table *) rotary_table;
+    if (!rt || 2 * rt->half > dim) { pi_set_error("pi_op_qkv_prepare: a rotation table over at most %d dimensions is required", dim); return -1; }
+    if (heads < 1 || kv_heads < 1 || heads % kv_heads) { pi_set_error("pi_op_qkv_prepare: %d query heads do not divide over %d key / value heads", heads, kv_heads); return -1; }
+    if (!dyn_dev || !cell_pos_dev) { pi_set_error("pi_op_qkv_prepare: the pass's cell table and the cells' position array are required"); return -1; }
+    if (pairing != PI_PAIR_HALVES && pairing != PI_PAIR_NEIGHBOURS) { pi_set_error("pi_op_qkv_prepare: pairing %d is unknown", pairing); return -1; }
+    if (norm_first && (!q_norm_w || !k_norm_w)) { pi_set_error("pi_op_qkv_prepare: norm weights are required"); return -1; }
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 8.0 * n_tok * ((double) heads * dim + (double) kv_heads * (dim + vdim)), k_qkv_prepare_any, dim3((unsigned) n_tok, (unsigned) (heads + 2 * kv_heads)), dim3(64), 0, (hipStream_t) stream,
+                 q, k, v, stride, q_norm_w, k_norm_w, eps, heads, kv_heads, dim, vdim, rt->cs, rt->half, rt->n_pos, norm_first, pairing, v_norm, pos_dev, q_out, q_out_stride, k_cache, v_cache, cell_pos_dev, dyn_dev, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+
 // ---- attention with sigmoid weights inside chunks ---------------------------------------------------------------------------------------------------------
 // grid (token, key / value head, split of its query heads): the workgroup serves the query heads of its key head (all of them in one workgroup unless they are very many or very wide).  The cells are walked 256 at a time; the visible ones of a round are compacted
 // in cell order (so that the sum has one order whatever the launch), their key rows staged in LDS 64 at a time.  Scores: thread (cell, query head); output: thread (query
@@ -153,7 +222,7 @@ static __device__ __forceinline__ void ca_stage(const float * __restrict__ cache
 template <int RPW>
 __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restrict__ q, int64_t qs, const float * __restrict__ kc, const float * __restrict__ vc, const int32_t * __restrict__ cell_pos,
                                                          const uint32_t * __restrict__ mask, const int32_t * __restrict__ pos, const float * __restrict__ hbias, const float * __restrict__ gate, int64_t gs, int gate_act,
-                                                         float scale, float out_mult, int chunk, int H, int G, int D, int V, int n_kv_arg, int tile, int hps, float * __restrict__ out, int64_t os, const int32_t * __restrict__ dyn,
+                                                         float scale, float out_mult, int weights, float softcap, int chunk, int H, int G, int D, int V, int n_kv_arg, int tile, int hps, float * __restrict__ out, int64_t os, const int32_t * __restrict__ dyn,
                                                          const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 5)) return;
     extern __shared__ float lds[];                // q [hpg][D] | key tile [tile][D + 1], then the value tile [tile][V] in the same place | weights [tile][hpg]
@@ -161,6 +230,9 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
     const int t = blockIdx.x, g = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int hs = blockIdx.z * hps, hpg = min(hps, H / G - hs), h0 = g * (H / G) + hs, DP = D + 1;        // this workgroup's query heads: hpg of them from h0 on (all of the key head's unless they are split over blockIdx.z)
     float * qsh = lds, * ksh = qsh + hpg * D, * wsh = ksh + tile * max(DP, V);
+    float * m_run = wsh + tile * hps, * l_run = m_run + hps, * f_run = l_run + hps;        // soft-max weights: per query head the running maximum, denominator, and the factor the sums so far take this tile
+    const bool soft = weights != PI_WEIGHTS_SIGMOID;
+    if (soft) for (int m = tid; m < hpg; m += 256) { m_run[m] = weights == PI_WEIGHTS_SOFTMAX_SINK ? 0.0f : -INFINITY; l_run[m] = weights == PI_WEIGHTS_SOFTMAX_SINK ? 1.0f : 0.0f; }      // (a sink: one more key of score 0 that has no value)
     const int n_kv = min(dyn ? dyn[1] : n_kv_arg, n_kv_arg);
     const int words = (n_kv_arg + 31) / 32;
     const uint32_t * mrow = mask + (int64_t) t * words;
@@ -207,9 +279,20 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
                 const float * kr = ksh + cc * DP, * qr = qsh + m * D;
                 float s = 0.0f;
                 for (int d = 0; d < D; d++) s = fmaf(qr[d], kr[d], s);
-                wsh[cc * hpg + m] = pm_sigmoid(s * scale + (hbias ? hbias[h0 + m] : 0.0f));
+                s = s * scale + (hbias ? hbias[h0 + m] : 0.0f);
+                if (soft && softcap > 0.0f) s = softcap * tanhf(s / softcap);
+                wsh[cc * hpg + m] = soft ? s : pm_sigmoid(s);
             }
             __syncthreads();
+            if (soft)                             // a wave per query head, a lane per cell of the tile (tile <= 64): new maximum, exponentials in the scores' place, denominator
+                for (int m = wave; m < hpg; m += 4) {
+                    const float sc = lane < nl ? wsh[lane * hpg + m] : -INFINITY;
+                    const float m_old = m_run[m], m_new = fmaxf(m_old, pi_wave_max(sc));
+                    const float e = lane < nl ? expf(sc - m_new) : 0.0f;
+                    const float sum = pi_lanes_sum<64>(e);
+                    if (lane < nl) wsh[lane * hpg + m] = e;
+                    if (lane == 0) { const float f = m_old == -INFINITY ? 0.0f : expf(m_old - m_new); m_run[m] = m_new; l_run[m] = fmaf(l_run[m], f, sum); f_run[m] = f; }
+                }
             // the value rows take the key tile's place: all their loads are in flight together (read one by one in the sum below, every row would cost a trip to memory)
             ca_stage<RPW>(vc, list + l0, nl, G, g, V, V, ksh, tid);
             __syncthreads();
@@ -218,7 +301,7 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
                 const int o = oi * 256 + tid;
                 if (o < n_out) {
                     const int m = o / V, vv = o % V;
-                    float a = acc[oi];
+                    float a = soft ? acc[oi] * f_run[m] : acc[oi];
                     for (int cc = 0; cc < nl; cc++) a = fmaf(wsh[cc * hpg + m], ksh[cc * V + vv], a);
                     acc[oi] = a;
                 }
@@ -232,7 +315,8 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
             const int m = o / V;
             float gt = gate ? gate[(int64_t) t * gs + h0 + m] : 1.0f;
             if (gate && gate_act == PI_ACT_SIGMOID) gt = pm_sigmoid(gt);
-            out[(int64_t) t * os + (int64_t) h0 * V + o] = acc[oi] * gt * out_mult;
+            const float den = soft ? l_run[m] : 1.0f;
+            out[(int64_t) t * os + (int64_t) h0 * V + o] = (soft ? (den > 0.0f ? acc[oi] / den : 0.0f) : acc[oi]) * gt * out_mult;
         }
     }
 }
@@ -240,19 +324,26 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
 extern "C" int pi_op_chunk_attention(const float * q, int64_t q_stride, const float * k_cache, const float * v_cache, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
                                      const float * head_bias_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int chunk, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv,
                                      float * out, int64_t out_stride, const int32_t * dyn_dev, void * stream) {
+    return pi_op_chunk_attention_ex(q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, gate_dev, gate_stride, gate_act, scale, out_mult, PI_WEIGHTS_SIGMOID, 0.0f, chunk, heads, kv_heads, dim, vdim,
+                                    n_tok, n_kv, out, out_stride, dyn_dev, stream);
+}
+extern "C" int pi_op_chunk_attention_ex(const float * q, int64_t q_stride, const float * k_cache, const float * v_cache, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
+                                        const float * head_bias_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int weights, float softcap, int chunk, int heads, int kv_heads,
+                                        int dim, int vdim, int n_tok, int n_kv, float * out, int64_t out_stride, const int32_t * dyn_dev, void * stream) {
     if (n_tok <= 0) return 0;
+    if (weights != PI_WEIGHTS_SIGMOID && weights != PI_WEIGHTS_SOFTMAX && weights != PI_WEIGHTS_SOFTMAX_SINK) { pi_set_error("pi_op_chunk_attention: weights of kind %d are unknown", weights); return -1; }
     if (heads < 1 || kv_heads < 1 || heads % kv_heads || dim < 1 || vdim < 1 || chunk < 0) { pi_set_error("pi_op_chunk_attention: %d query heads over %d key / value heads, sizes %d / %d, chunk %d", heads, kv_heads, dim, vdim, chunk); return -1; }
     int hpg = heads / kv_heads, splits = 1;                            // query heads of a key head that one workgroup serves: all of them, unless their outputs or the LDS plan say otherwise
     while (hpg > 1 && (hpg * vdim > 256 * CA_MAXOUT || (size_t) hpg * dim * sizeof(float) > 24 * 1024)) { splits *= 2; hpg = (heads / kv_heads + splits - 1) / splits; }
     int tile = CA_TILE;
-    auto lds_of = [&](int tl) { return ((size_t) hpg * dim + (size_t) tl * std::max(dim + 1, vdim) + (size_t) tl * hpg) * sizeof(float); };
+    auto lds_of = [&](int tl) { return ((size_t) hpg * dim + (size_t) tl * std::max(dim + 1, vdim) + (size_t) tl * hpg + (size_t) 3 * hpg) * sizeof(float); };
     while (tile > 4 && lds_of(tile) > 60 * 1024) tile >>= 1;
     const size_t lds = lds_of(tile);
     if (hpg * vdim > 256 * CA_MAXOUT || lds > 60 * 1024) { pi_set_error("pi_op_chunk_attention: %d query heads per key head of sizes %d / %d are beyond the kernel (LDS %zu bytes)", hpg, dim, vdim, lds); return -1; }
     const int acct = pi_account_n_kv() > 0 ? pi_account_n_kv() : n_kv;
     const double visible = chunk > 0 ? std::min(acct, chunk) : acct;
 #define CA_GO(R)     PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), 4.0 * visible * kv_heads * (dim + vdim) + 4.0 * n_tok * heads * (dim + vdim), k_chunk_attention<R>, dim3((unsigned) n_tok, (unsigned) kv_heads, (unsigned) ((heads / kv_heads + hpg - 1) / hpg)), dim3(256), lds, \
-                 (hipStream_t) stream, q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, gate_dev, gate_stride, gate_act, scale, out_mult, chunk, heads, kv_heads, dim, vdim, n_kv, tile, hpg, out, out_stride, \
+                 (hipStream_t) stream, q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, gate_dev, gate_stride, gate_act, scale, out_mult, weights, softcap, chunk, heads, kv_heads, dim, vdim, n_kv, tile, hpg, out, out_stride, \
                  dyn_dev, pi_abort_word());
     CA_GO(4);                                                          // (deeper rounds were measured for single tokens: no gain, the registers they take cost as much as the trips they save)
 #undef CA_GO

@@ -4,7 +4,10 @@ same width, depth and head count with Q8_0 weights, the densest quantised type t
 `bench.py --compare-hybrid [SIZE,...]` prints one JSON line per size; bench.py's default workload and line are untouched.
 
 `bench.py --compare-parallel [SIZE,...]` does the same for the Vikarax design (parallel mixer: chunked sigmoid attention beside a selective recurrence, gated experts with a
-shared one) beside the engine's closest model, which is Fasovik at the same width, depth, head sizes and expert sizes."""
+shared one) beside the engine's closest model, which is Fasovik at the same width, depth, head sizes and expert sizes.
+
+`bench.py --compare-postnorm [SIZE,...]`: the Rafusun design (delta-rule layers and attention + time-mix layers in turn, a gated dense feed-forward, the norm after the sum) beside the
+closest model, which is Vikarax at the same width, depth, attention sizes and with a dense feed-forward of the same width."""
 import ctypes as C
 import json
 import os
@@ -109,7 +112,8 @@ def write_random_tensors(folder, cfg, shapes, ones=(), seed=1):
     return folder
 
 
-def write_vikarax(folder, size, seed=1):
+def write_vikarax(folder, size, seed=1, dense_ff=0):
+    """dense_ff > 0: a dense feed-forward of that width in place of the routed experts"""
     width, n_layer, heads, dim, vdim, _, n_exp, _, top, ff, vocab = SIZES[size]
     kv_heads, rot, chunk, r_heads, r_vdim, state, groups, g_count, g_keep, shared = VIKARAX[size]
     inner, gn = r_heads * r_vdim, groups * state
@@ -118,6 +122,8 @@ def write_vikarax(folder, size, seed=1):
         mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": n_exp, "top": top, "groups": {"count": g_count, "keep": g_keep}}, "shared": {"ff": shared}}
         left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "rot": {"dims": rot, "base": 10000.0}, "mask": {"size": chunk}}
         right = {"heads": r_heads, "vdim": r_vdim, "state": state, "groups": groups, "conv": 4, "norm_groups": groups}
+        if dense_ff:
+            mlp = {"kind": "dense", "ff": dense_ff}
         layers.append({"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 0.7, "right_scale": 0.7}, "mlp": mlp})
         p = "l%d." % i
         for n in ("norm1", "norm1b", "norm2", "norm2b"):
@@ -129,12 +135,46 @@ def write_vikarax(folder, size, seed=1):
         q = p + "mix.right."
         shapes.update({q + "in": (2 * inner + 2 * gn + r_heads, width), q + "conv": (inner + 2 * gn, 4), q + "conv.b": (inner + 2 * gn,), q + "dt_bias": (r_heads,), q + "A_log": (r_heads,),
                        q + "D": (r_heads,), q + "norm": (inner,), q + "o": (width, inner)})
+        if dense_ff:
+            shapes.update({p + "mlp.up": (dense_ff, width), p + "mlp.down": (width, dense_ff)})
+            continue
         shapes[p + "mlp.router"] = (n_exp, width)
         for e in ["e%d" % e for e in range(n_exp)] + ["shared"]:
             f = shared if e == "shared" else ff
             shapes.update({p + "mlp.%s.gate" % e: (f, width), p + "mlp.%s.up" % e: (f, width), p + "mlp.%s.down" % e: (width, f)})
     cfg = {"architecture": "Vikarax", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "logit_softcap": 30.0, "layers": layers}
     return write_random_tensors(folder, cfg, shapes, ones=("norm", "norm1", "norm2", "norm1b", "norm2b", "dwa", ".D"), seed=seed)
+
+
+def write_rafusun(folder, size, seed=1):
+    """layers in turn: a delta-rule mixer without a feed-forward, then attention + time mixing with a gated dense feed-forward (attention sizes as the Vikarax model of this size)"""
+    width, n_layer, heads, dim, vdim, _, _, _, _, ff, vocab = SIZES[size]
+    kv_heads, rot, chunk, r_heads, r_vdim, _, _, _, _, _ = VIKARAX[size]
+    dense_ff, rank = 4 * ff, 64
+    layers, shapes = [], {"embed": (vocab, width), "bigram": (65537, width), "head": (vocab, width), "final.norm": (width,)}
+    for i in range(n_layer):
+        p = "l%d." % i
+        shapes[p + "norm1"] = shapes[p + "ls1"] = (width,)
+        if i % 2 == 0:
+            layers.append({"type": "channel_delta", "mixer": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "conv": 4}, "mlp": None})
+            q = p + "mix."
+            shapes.update({q + "q": (kv_heads * dim, width), q + "k": (kv_heads * dim, width), q + "v": (heads * vdim, width), q + "q.conv": (kv_heads * dim, 4), q + "k.conv": (kv_heads * dim, 4),
+                           q + "v.conv": (heads * vdim, 4), q + "b": (heads, width), q + "A_log": (heads,), q + "dt_bias": (heads * dim,), q + "a1": (rank, width), q + "a2": (heads * dim, rank),
+                           q + "g1": (rank, width), q + "g2": (heads * vdim, rank), q + "norm": (vdim,), q + "o": (width, heads * vdim)})
+            continue
+        left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "softcap": 30.0, "rot": {"dims": rot, "base": 10000.0}, "mask": {"size": chunk}}
+        layers.append({"type": "parallel", "mixer": {"left": left, "right": {"heads": r_heads, "dim": r_vdim}}, "mlp": {"kind": "dense", "ff": dense_ff}})
+        inner = r_heads * r_vdim
+        q = p + "mix.left."
+        shapes.update({q + "q": (heads * dim, width), q + "k": (kv_heads * dim, width), q + "v": (kv_heads * vdim, width), q + "o": (width, heads * vdim), q + "out": (width,)})
+        q = p + "mix.right."
+        shapes.update({q + "mu." + n: (width,) for n in "rkvgw"})
+        shapes.update({q + n: (inner, width) for n in "rkvg"})
+        shapes.update({q + "w1": (rank, width), q + "w2": (inner, rank), q + "w0": (inner,), q + "u": (r_heads, r_vdim), q + "norm": (inner,), q + "o": (width, inner), q + "out": (width,)})
+        shapes.update({p + "norm2": (width,), p + "ls2": (width,), p + "mlp.gate": (dense_ff, width), p + "mlp.up": (dense_ff, width), p + "mlp.down": (width, dense_ff)})
+    cfg = {"architecture": "Rafusun", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "postln_alpha": 2.0, "embedding": {"scale": 1.0, "bigram": {"buckets": 65536, "mul_prev": 8191, "mul_cur": 31}},
+           "layers": layers}
+    return write_random_tensors(folder, cfg, shapes, ones=("norm", "norm1", "norm2", "ls1", "ls2", ".out"), seed=seed)
 
 
 class KtRow(C.Structure):          # struct pi_kt_row (include/pipeinfer_ops.h)
@@ -225,6 +265,28 @@ def main_parallel(sizes, cache, n_prompt=512, n_decode=64):
     return 0
 
 
+def main_postnorm(sizes, cache, n_prompt=512, n_decode=64):
+    """Rafusun beside Vikarax (dense feed-forward of the same width) at equal sizes; one JSON line per size"""
+    lib = L.load()
+    L.check(lib.pi_device_init(0), "pi_device_init")
+    for size in sizes:
+        width, n_layer, heads, dim, vdim, _, _, _, _, ff, vocab = SIZES[size]
+        kv_heads, rot, chunk, r_heads, r_vdim, state, groups, _, _, _ = VIKARAX[size]
+        raf, vik = os.path.join(cache, "rafusun-" + size), os.path.join(cache, "vikarax-dense-" + size)
+        if not os.path.exists(os.path.join(raf, "model.safetensors")):
+            write_rafusun(raf, size)
+        if not os.path.exists(os.path.join(vik, "model.safetensors")):
+            write_vikarax(vik, size, dense_ff=4 * ff)
+        out = {"size": size, "config": {"width": width, "layers": n_layer, "heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "rot_dims": rot, "chunk": chunk, "conv": 4, "low_rank": 64,
+                                       "time_mix": {"heads": r_heads, "dim": r_vdim}, "vikarax_recurrence": {"heads": r_heads, "vdim": r_vdim, "state": state, "groups": groups}, "ff": 4 * ff,
+                                       "vocab": vocab, "n_prompt": n_prompt, "n_decode": n_decode},
+               "rafusun_bf16": measure(lib, raf, n_prompt, n_decode, True),
+               "vikarax_dense_bf16": measure(lib, vik, n_prompt, n_decode, True), "data": "synthetic", "hbm_peak": HBM_PEAK}
+        print(json.dumps(out))
+        sys.stdout.flush()
+    return 0
+
+
 def main(sizes, cache, n_prompt=512, n_decode=64):
     lib = L.load()
     L.check(lib.pi_device_init(0), "pi_device_init")
@@ -253,7 +315,7 @@ def run_phase(design, size, phase, cache, n_prompt=512, n_decode=64):
     L.check(lib.pi_device_init(0), "pi_device_init")
     folder = os.path.join(cache, "%s-%s" % (design, size))
     if not os.path.exists(os.path.join(folder, "model.safetensors")):
-        (write_vikarax if design == "vikarax" else write_fasovik)(folder, size)
+        {"vikarax": write_vikarax, "fasovik": write_fasovik, "rafusun": write_rafusun}[design](folder, size)
     model = LL.Model(folder)
     ctx = LL.Context(model, n_ctx=n_prompt + n_decode + 64, n_batch=n_prompt)
     ctx.set_precision(False)
@@ -274,7 +336,7 @@ def run_phase(design, size, phase, cache, n_prompt=512, n_decode=64):
 if __name__ == "__main__":
     import argparse
     ap = argparse.ArgumentParser(description="one phase of one folder-described design at one size (for `rocprofv3 --kernel-trace --stats -- python3 -m pipeinfer_amd.tools.hybrid_bench ...`)")
-    ap.add_argument("--design", choices=["vikarax", "fasovik"], required=True)
+    ap.add_argument("--design", choices=["vikarax", "fasovik", "rafusun"], required=True)
     ap.add_argument("--size", choices=sorted(SIZES), default="w2048")
     ap.add_argument("--phase", choices=["prefill", "decode"], required=True)
     ap.add_argument("--cache", default=os.environ.get("PIPEINFER_CACHE", "/tmp/pipeinfer_models"))

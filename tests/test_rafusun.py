@@ -1,0 +1,691 @@
+"""The Rafusun design (the norm after the sum with layer scales, a hashed pair embedding, a delta-rule mixer with a decay per key channel behind short convolutions, chunked
+soft-max attention with a sink and capped scores beside time mixing with a token shift, a gated dense feed-forward) on the engine, held to the plain numpy restatement in
+tests/rafusun_oracle.py: every mechanism alone through its operator, then whole models through llama_decode — prompts against token-by-token decoding, portions down to two
+tokens, batches of unequal requests, cells and state slots freed and used again, keys at the borders of chunks, long decoding, greedy generation, the trace runner.  Models are
+small, random and made here; sizes are chosen so that nothing that could be mixed up is equal."""
+import ctypes as C
+import json
+import os
+
+import numpy as np
+import pytest
+
+from pipeinfer_amd import lib as L, llama as LL
+from tests import rafusun_oracle as O
+
+BF16 = 30
+F = 1 << 30                                    # "this sequence starts from nothing" on the first token of a run (rec words)
+NONE, SILU, SIGMOID, TANH, GELU = 0, 1, 2, 4, 5
+DELTA, BONUS = 0, 1
+
+
+def rel_rms(got, want):
+    d = np.asarray(got, np.float64) - np.asarray(want, np.float64)
+    return float(np.sqrt((d * d).mean()) / (np.sqrt((np.asarray(want, np.float64) ** 2).mean()) + 1e-30))
+
+
+def logit_err(got, want):
+    d = np.asarray(got, np.float64) - want
+    d = d - d.mean(-1, keepdims=True)
+    return np.sqrt((d * d).mean(-1)) / (want - want.mean(-1, keepdims=True)).std()
+
+
+TOL = {True: 3e-4, False: 4e-2}          # exact (fp32) / serving precision (bfloat16 matrix inputs)
+
+VOCAB = 83
+# layer mixes: the default one, the values another model may make equal or one, wide heads, and the sizes that straddle the kernels' tiles
+VARIANTS = {
+    "mixed": None,
+    "edges": [O.delta_layer(heads=1, kv_heads=1, dim=3, vdim=3, conv=1, decay_rank=1, gate_rank=1, mlp=O.dense_mlp(1)),
+              O.parallel_layer(heads=1, kv_heads=1, dim=2, vdim=1, chunk=1, rot_dims=2, softcap=None, r_heads=1, r_dim=1, decay_rank=1, mlp=None),
+              O.parallel_layer(heads=2, kv_heads=2, dim=4, vdim=4, chunk=None, rot_dims=None, r_heads=1, r_dim=5, mlp=O.dense_mlp(9)),
+              O.delta_layer(heads=3, kv_heads=3, dim=4, vdim=4, conv=2, mlp=None)],
+    "wide_heads": [O.delta_layer(heads=2, kv_heads=1, dim=40, vdim=70, conv=5, decay_rank=6, gate_rank=5, mlp=None),
+                   O.parallel_layer(heads=6, kv_heads=2, dim=72, vdim=66, chunk=19, rot_dims=72, r_heads=2, r_dim=36, decay_rank=8, mlp=O.dense_mlp(50)),
+                   O.delta_layer(heads=4, kv_heads=2, dim=66, vdim=10, conv=4, mlp=O.dense_mlp(33))],
+    "only_parallel": [O.parallel_layer(mlp=None), O.parallel_layer(heads=3, kv_heads=1, dim=8, vdim=4, chunk=4, rot_dims=6, r_heads=2, r_dim=8, mlp=O.dense_mlp(12))],
+    "only_delta": [O.delta_layer(mlp=O.dense_mlp(11)), O.delta_layer(heads=4, kv_heads=1, dim=9, vdim=2, conv=8, mlp=None)],
+}
+
+
+def small_model(seed=0, width=40, vocab=VOCAB, layers=None, **kw):
+    rng = np.random.default_rng(seed)
+    layers = layers or [O.delta_layer(mlp=None),
+                        O.parallel_layer(mlp=O.dense_mlp(24)),
+                        O.delta_layer(heads=4, kv_heads=2, dim=5, vdim=7, conv=4, decay_rank=4, gate_rank=3, mlp=O.dense_mlp(13)),
+                        O.parallel_layer(heads=2, kv_heads=2, dim=10, vdim=4, chunk=16, rot_dims=2, r_heads=2, r_dim=7, decay_rank=3, mlp=None)]
+    return O.random_model(rng, vocab, width, layers, **kw)
+
+
+def write(folder, m):
+    O.write_model(folder, m["config"], {k: v.astype(np.float32) for k, v in m["tensors"].items()})
+
+
+class Engine:
+    def __init__(self, tmp_path, model, n_ctx=256, n_batch=64, exact=True, slots=4, name="m"):
+        folder = os.path.join(str(tmp_path), name)
+        write(folder, model)
+        self.model = LL.Model(folder)
+        self.ctx = LL.Context(self.model, n_ctx=n_ctx, n_batch=n_batch)
+        self.ctx.set_state_slots(slots)
+        self.ctx.set_precision(exact)
+
+    def close(self):
+        self.ctx.free()
+        self.model.free()
+
+
+# ---- without a GPU ---------------------------------------------------------------------------------------------------------------
+def test_model_folder_is_read_and_described(tmp_path):
+    m = small_model()
+    folder = str(tmp_path / "m")
+    write(folder, m)
+    mod = LL.Model(folder)
+    assert mod.n_vocab == VOCAB
+    buf = C.create_string_buffer(64)
+    mod.lib.llama_model_desc.argtypes = [C.c_void_p, C.c_char_p, C.c_size_t]
+    mod.lib.llama_model_desc(mod.h, buf, 64)
+    assert buf.value.lower().startswith(b"rafusun")
+    mod.free()
+    for name, layers in VARIANTS.items():                          # descriptions without chunks, a rotation, a cap or a feed-forward are read as well
+        if layers:
+            mv = small_model(seed=1, layers=layers, width=64 if name == "wide_heads" else 40)
+            write(str(tmp_path / name), mv)
+            LL.Model(str(tmp_path / name)).free()
+
+
+@pytest.mark.parametrize("breakage", ["type", "kv_heads", "delta_kv_heads", "rot", "kind", "alpha", "conv", "tensor"])
+def test_a_wrong_description_is_refused(tmp_path, breakage):
+    m = small_model()
+    cfg = json.loads(json.dumps(m["config"]))
+    tensors = dict(m["tensors"])
+    if breakage == "type":
+        cfg["layers"][0]["type"] = "serial"
+    elif breakage == "kv_heads":
+        cfg["layers"][1]["mixer"]["left"]["kv_heads"] = 3
+    elif breakage == "delta_kv_heads":
+        cfg["layers"][2]["mixer"]["kv_heads"] = 3
+    elif breakage == "rot":
+        cfg["layers"][1]["mixer"]["left"]["rot"]["dims"] = 5
+    elif breakage == "kind":
+        cfg["layers"][1]["mlp"]["kind"] = "moe"
+    elif breakage == "alpha":
+        del cfg["postln_alpha"]
+    elif breakage == "conv":
+        cfg["layers"][0]["mixer"]["conv"] = 0
+    elif breakage == "tensor":
+        del tensors["l0.mix.a1"]
+    folder = str(tmp_path / "bad")
+    O.write_model(folder, cfg, {k: v.astype(np.float32) for k, v in tensors.items()})
+    with pytest.raises(L.PipeInferError):
+        LL.Model(folder)
+
+
+def test_oracle_mechanisms_behave_as_stated():
+    """the restatement itself: a rotation of neighbours that keeps lengths and depends on the distance only, the chunk border, the sink, a delta rule that stores and replaces a value, a bonus
+    that only the token itself sees, the pair table's rows"""
+    rng = np.random.default_rng(3)
+    v = rng.standard_normal(8)
+    r = O.rotate_pairs(v, 11, 6, 100.0)
+    assert np.isclose(np.linalg.norm(r), np.linalg.norm(v)) and np.array_equal(r[6:], v[6:]) and np.isclose(np.hypot(r[0], r[1]), np.hypot(v[0], v[1]))
+    a, b = rng.standard_normal(4), rng.standard_normal(4)
+    assert np.isclose(O.rotate_pairs(a, 9, 4, 30.0) @ O.rotate_pairs(b, 5, 4, 30.0), O.rotate_pairs(a, 104, 4, 30.0) @ O.rotate_pairs(b, 100, 4, 30.0))
+    m = small_model(seed=3, layers=[O.parallel_layer(chunk=4, mlp=None)])
+    T, c = m["tensors"], m["config"]["layers"][0]["mixer"]["left"]
+    hs = rng.standard_normal((6, 40))
+    st = {}
+    outs = [O.softmax_attention_step(T, "l0.mix.left.", c, 1e-5, hs[i], i, st) for i in range(6)]
+    alone = O.softmax_attention_step(T, "l0.mix.left.", c, 1e-5, hs[4], 4, {})        # positions 0..3 are one chunk, 4 starts the next: token 4 sees itself only
+    assert np.allclose(alone, outs[4]) and not np.allclose(outs[5], O.softmax_attention_step(T, "l0.mix.left.", c, 1e-5, hs[5], 5, {}))
+    big = dict(c, scale=0.0, softcap=None)                                               # all scores 0: one key shares the mass with the sink, p = 1 / 2
+    T2 = dict(T)
+    T2["l0.mix.left.o"] = np.eye(40, c["heads"] * c["vdim"])
+    o = O.softmax_attention_step(T2, "l0.mix.left.", big, 1e-5, hs[0], 0, {})
+    vrow = (T["l0.mix.left.v"] @ hs[0]).reshape(c["kv_heads"], c["vdim"])
+    assert np.allclose(o[:c["vdim"]], 0.5 * vrow[0])
+    # delta rule with g = 1, beta = 1 and unit keys: writing v1 under k, then v2 under the same k, leaves exactly v2 under k
+    S = np.zeros((3, 2))
+    k = np.array([0.0, 1.0, 0.0])
+    for val in (np.array([1.0, 2.0]), np.array([-3.0, 5.0])):
+        S = S + np.outer(k, val - S.T @ k)
+    assert np.allclose(S.T @ k, [-3.0, 5.0])
+    cfg = m["config"]["embedding"]["bigram"]
+    assert np.array_equal(O.embed(m, 7, None), T["embed"][7] * m["config"]["embedding"]["scale"] + T["bigram"][cfg["buckets"]])
+    assert np.array_equal(O.embed(m, 7, 80), T["embed"][7] * m["config"]["embedding"]["scale"] + T["bigram"][(80 * cfg["mul_prev"] + 7 * cfg["mul_cur"]) % cfg["buckets"]])
+
+
+# ---- operators alone ---------------------------------------------------------------------------------------------------------------
+def gpu():
+    from tests import gpu_util as U
+    return U, U.init()
+
+
+def upload_bf16(lib, w):
+    u = (np.ascontiguousarray(w, np.float32).view(np.uint32) >> 16).astype(np.uint16)
+    h = lib.pi_weight_upload(BF16, w.shape[1], w.shape[0], u.ctypes.data_as(C.c_void_p), None)
+    assert h, lib.pi_last_error()
+    return h
+
+
+def pack_mask(vis, n_kv):
+    words = (n_kv + 31) // 32
+    m = np.zeros((vis.shape[0], words), np.uint32)
+    for t, j in zip(*np.nonzero(vis)):
+        m[t, j >> 5] |= np.uint32(1 << (j & 31))
+    return m
+
+
+@pytest.mark.gpu
+def test_embedding_adds_the_pair_row():
+    U, lib = gpu()
+    rng = np.random.default_rng(1)
+    table, table2 = O.bf16_round(rng.standard_normal((20, 37)).astype(np.float32)), O.bf16_round(rng.standard_normal((12, 37)).astype(np.float32))
+    toks, rows = np.array([3, 19, 0, 3], np.int32), np.array([11, 0, 5, 5], np.int32)
+    w, w2 = upload_bf16(lib, table), upload_bf16(lib, table2)
+    td, rd, od = U.Dev(toks), U.Dev(rows), U.Dev(nbytes=4 * 4 * 37)
+    L.check(lib.pi_op_embed_pair(w, td.ptr, 4, 2.5, w2, rd.ptr, od.ptr, None))
+    assert rel_rms(od.get(np.float32, (4, 37)), table[toks].astype(np.float64) * 2.5 + table2[rows]) < 1e-7
+    lib.pi_weight_free(w)
+    lib.pi_weight_free(w2)
+
+
+@pytest.mark.gpu
+def test_dense_epilogues_tanh_and_gelu():
+    U, lib = gpu()
+    rng = np.random.default_rng(2)
+    W, x = O.bf16_round(rng.standard_normal((11, 24)).astype(np.float32)), (rng.standard_normal((5, 24)) * 2).astype(np.float32)
+    w, xd, od = upload_bf16(lib, W), U.Dev(x), U.Dev(nbytes=4 * 5 * 11)
+    L.check(lib.pi_op_dense(w, xd.ptr, 24, 5, od.ptr, 11, GELU, 6, TANH, 1, None))
+    z = x.astype(np.float64) @ W.T.astype(np.float64)
+    want = np.concatenate([O.gelu_tanh(z[:, :6]), np.tanh(z[:, 6:])], axis=1)
+    assert rel_rms(od.get(np.float32, (5, 11)), want) < 2e-6
+    lib.pi_weight_free(w)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n", [5, 96, 300, 1000, 2100])
+def test_sublayer_end_with_one_and_two_inputs(n):
+    """layer scale, + alpha x, norm; the mean of two normed branches in front; the second norm behind; in place"""
+    U, lib = gpu()
+    rng = np.random.default_rng(n)
+    T = 4
+    a, b, x = ((rng.standard_normal((T, n + 3)) * 3).astype(np.float32) for _ in range(3))
+    wa, wb, ls, w, wn = (rng.standard_normal(n).astype(np.float32) for _ in range(5))
+    ad, bd, xd, od, nd = U.Dev(a), U.Dev(b), U.Dev(x), U.Dev(nbytes=4 * T * n), U.Dev(nbytes=4 * T * n)
+    ws = [U.Dev(v) for v in (wa, wb, ls, w, wn)]
+    a64, b64, x64 = a[:, :n].astype(np.float64), b[:, :n].astype(np.float64), x[:, :n].astype(np.float64)
+    L.check(lib.pi_op_rms_post(ad.ptr, n + 3, None, None, 0, None, 1.0, ws[2].ptr, xd.ptr, n + 3, 1.7, ws[3].ptr, 1e-3, n, T, od.ptr, n, None, None, 0, None))
+    one = np.stack([O.unit_rms(1.7 * x64[t] + ls * a64[t], 1e-3) * w for t in range(T)])
+    assert rel_rms(od.get(np.float32, (T, n)), one) < 2e-6
+    L.check(lib.pi_op_rms_post(ad.ptr, n + 3, None, None, 0, None, 1.0, None, xd.ptr, n + 3, -0.5, ws[3].ptr, 1e-3, n, T, od.ptr, n, None, None, 0, None))       # no layer scale
+    assert rel_rms(od.get(np.float32, (T, n)), np.stack([O.unit_rms(-0.5 * x64[t] + a64[t], 1e-3) * w for t in range(T)])) < 2e-6
+    two = np.stack([O.unit_rms(1.7 * x64[t] + ls * 0.5 * (O.unit_rms(a64[t], 1e-3) * wa + O.unit_rms(b64[t], 1e-3) * wb), 1e-3) * w for t in range(T)])
+    nxt = np.stack([O.unit_rms(two[t], 1e-3) * wn for t in range(T)])
+    L.check(lib.pi_op_rms_post(ad.ptr, n + 3, ws[0].ptr, bd.ptr, n + 3, ws[1].ptr, 0.5, ws[2].ptr, xd.ptr, n + 3, 1.7, ws[3].ptr, 1e-3, n, T, xd.ptr, n + 3, ws[4].ptr, nd.ptr, n, None))     # in place
+    assert rel_rms(xd.get(np.float32, (T, n + 3))[:, :n], two) < 3e-6 and rel_rms(nd.get(np.float32, (T, n)), nxt) < 4e-6
+    assert np.array_equal(xd.get(np.float32, (T, n + 3))[:, n:], x[:, n:])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,n_mix", [(7, 1), (300, 5), (64, 3)])
+def test_token_shift_over_sequences_and_passes(n, n_mix):
+    """three sequences, passes of 1..40 tokens (both entries of the operator), a slot handed to a new owner over the old owner's row"""
+    U, lib = gpu()
+    rng = np.random.default_rng(n)
+    mu = rng.uniform(0, 1, (n_mix, n)).astype(np.float32)
+    slots = 3
+    state = U.Dev((rng.standard_normal((slots, n)) * 50).astype(np.float32))               # (garbage: a fresh slot must not read it)
+    md = U.Dev(mu)
+    prev = {}
+    plan = [[(0, 5, True), (2, 1, True)], [(2, 40, False), (0, 2, False)], [(1, 3, True)], [(0, 1, False), (1, 1, False), (2, 1, False)], [(1, 36, True), (0, 33, False)]]
+    for step in plan:
+        T = sum(c for _, c, _ in step)
+        h = rng.standard_normal((T, n + 1)).astype(np.float32)
+        rec, want, at = [], np.zeros((T, n_mix, n)), 0
+        for slot, count, fresh in step:
+            if fresh:
+                prev[slot] = np.zeros(n)
+            for i in range(count):
+                rec.append(slot | (F if fresh and i == 0 else 0))
+                cur = h[at, :n].astype(np.float64)
+                want[at] = cur + (prev[slot] - cur) * mu
+                prev[slot] = cur
+                at += 1
+        hd, rd, od = U.Dev(h), U.Dev(np.array(rec, np.int32)), U.Dev(nbytes=4 * T * (n_mix * n + 2))
+        L.check(lib.pi_op_token_shift(hd.ptr, n + 1, n, md.ptr, n_mix, state.ptr, rd.ptr, T, od.ptr, n_mix * n + 2, None))
+        got = od.get(np.float32, (T, n_mix * n + 2))[:, :n_mix * n].reshape(T, n_mix, n)
+        assert rel_rms(got, want) < 1e-6
+    st = state.get(np.float32, (slots, n))
+    for slot in range(3):
+        assert rel_rms(st[slot], prev[slot]) < 1e-7
+
+
+def recurrence_ref(rule, q, k, v, g, beta, bonus, S):
+    """one head, one token, float64: returns the output and the new state"""
+    if rule == DELTA:
+        S = S * g[:, None]
+        u = beta * (v - S.T @ k)
+        S = S + np.outer(k, u)
+        return S.T @ q, S
+    kv = np.outer(k, v)
+    return (S + bonus[:, None] * kv).T @ q, g[:, None] * S + kv
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D,V", [(2, 1, 6, 5), (1, 1, 40, 70), (4, 2, 33, 8), (3, 3, 130, 20), (2, 2, 8, 300), (1, 1, 1, 1)])
+@pytest.mark.parametrize("rule", [DELTA, BONUS])
+def test_channel_recurrence_rules_decays_and_passes(H, G, D, V, rule):
+    """both rules with every way of forming the decays, unit vectors and beta, grouped q / k heads, several sequences per pass, carried and fresh states, passes longer than a tile"""
+    U, lib = gpu()
+    rng = np.random.default_rng(H * 100 + D + V + rule)
+    slots = 3
+    states = {s: None for s in range(slots)}
+    sd = U.Dev((rng.standard_normal((slots, H, D, V)) * 9).astype(np.float32))
+    dbias, a_log, bonus = (rng.standard_normal(H * D) - 1).astype(np.float32), (rng.standard_normal(H) * 0.5).astype(np.float32), rng.standard_normal((H, D)).astype(np.float32)
+    dbd, ald, bod = U.Dev(dbias), U.Dev(a_log), U.Dev(bonus)
+    plan = [(1, [(1, 4, True)]), (2, [(0, 3, True), (1, 2, False)]), (0, [(2, 37, True), (0, 1, False)]), (2, [(1, 1, False), (0, 35, False), (2, 1, False)])]
+    for mode, step in plan:
+        T = sum(c for _, c, _ in step)
+        q, k = rng.standard_normal((T, G * D + 1)).astype(np.float32), rng.standard_normal((T, G * D + 2)).astype(np.float32)
+        v, raw, braw = rng.standard_normal((T, H * V)).astype(np.float32), rng.standard_normal((T, H * D + 3)).astype(np.float32), rng.standard_normal((T, H + 1)).astype(np.float32)
+        if mode == 0:
+            raw = rng.uniform(0.3, 1.0, raw.shape).astype(np.float32)
+        unit = rule == DELTA
+        if not unit:
+            q, k = q * 0.4, k * 0.4
+        rec, want, at = [], np.zeros((T, H, V)), 0
+        for slot, count, fresh in step:
+            if fresh:
+                states[slot] = np.zeros((H, D, V))
+            for i in range(count):
+                rec.append(slot | (F if fresh and i == 0 else 0))
+                for h in range(H):
+                    j = h // (H // G)
+                    qh, kh = q[at, j * D:(j + 1) * D].astype(np.float64), k[at, j * D:(j + 1) * D].astype(np.float64)
+                    if unit:
+                        qh, kh = O.unit_length(qh) * 0.7, O.unit_length(kh)
+                    r = raw[at, h * D:(h + 1) * D].astype(np.float64)
+                    g = r if mode == 0 else np.exp(-np.exp(r + dbias[h * D:(h + 1) * D])) if mode == 1 else np.exp(-np.exp(a_log[h]) * O.softplus(r + dbias[h * D:(h + 1) * D]))
+                    want[at, h], states[slot][h] = recurrence_ref(rule, qh, kh, v[at, h * V:(h + 1) * V].astype(np.float64), g, O.sigmoid(braw[at, h]), bonus[h].astype(np.float64), states[slot][h])
+                at += 1
+        qd, kd, vd, rd, bd, rc, od = U.Dev(q), U.Dev(k), U.Dev(v), U.Dev(raw), U.Dev(braw), U.Dev(np.array(rec, np.int32)), U.Dev(nbytes=4 * T * (H * V + 1))
+        L.check(lib.pi_op_channel_recurrence(rule, qd.ptr, G * D + 1, kd.ptr, G * D + 2, vd.ptr, H * V, rd.ptr, H * D + 3, mode, dbd.ptr, ald.ptr, bd.ptr if rule == DELTA else None, H + 1,
+                                             bod.ptr if rule == BONUS else None, int(unit), 0.7 if unit else 1.0, H, G, D, V, sd.ptr, rc.ptr, T, slots, od.ptr, H * V + 1, None))
+        got = od.get(np.float32, (T, H * V + 1))[:, :H * V].reshape(T, H, V)
+        assert rel_rms(got, want) < 2e-5, (mode, step)
+    st = sd.get(np.float32, (slots, H, D, V))
+    for s in range(slots):
+        assert rel_rms(st[s], states[s]) < 2e-5
+
+
+@pytest.mark.gpu
+def test_delta_rule_keeps_a_far_value_and_replaces_it():
+    """a value written under one key 300 tokens back (decays of one, other keys orthogonal) is read back exactly; written again, the new value replaces the old one"""
+    U, lib = gpu()
+    D, V, T = 8, 4, 320
+    k = np.zeros((T, D), np.float32)
+    k[:, 1] = 1.0
+    k[0, :] = 0.0
+    k[0, 5] = 1.0                                                       # the far key: dimension 5, never used again until the end
+    k[T - 1, :] = 0.0
+    k[T - 1, 5] = 1.0
+    q = k.copy()
+    v = np.random.default_rng(0).standard_normal((T, V)).astype(np.float32)
+    raw, braw = np.ones((T, D), np.float32), np.full((T, 1), 30.0, np.float32)           # g = 1 (mode 0), beta = sigmoid(30) = 1
+    rec = np.zeros(T, np.int32)
+    rec[0] |= F
+    sd, od = U.Dev(np.full((1, 1, D, V), 7.0, np.float32)), U.Dev(nbytes=4 * T * V)
+    devs = [U.Dev(a) for a in (q, k, v, raw, braw, rec)]
+    L.check(lib.pi_op_channel_recurrence(DELTA, devs[0].ptr, D, devs[1].ptr, D, devs[2].ptr, V, devs[3].ptr, D, 0, None, None, devs[4].ptr, 1, None, 1, 1.0, 1, 1, D, V, sd.ptr, devs[5].ptr, T, 1, od.ptr, V, None))
+    got = od.get(np.float32, (T, V))
+    assert np.allclose(got[0], v[0], atol=1e-5) and np.allclose(got[T - 2], v[T - 2], atol=1e-5)
+    assert np.allclose(got[T - 1], v[T - 1], atol=1e-5)                 # the token's own write is what it reads ...
+    S = sd.get(np.float32, (D, V))
+    assert np.allclose(S[5], v[T - 1], atol=1e-5) and np.allclose(S[1], v[T - 2], atol=1e-5)      # ... and the far row held v[0] until then (S[5] was replaced, not summed)
+    devs[4] = U.Dev(np.full((T, 1), -30.0, np.float32))                  # beta = 0: nothing is ever written, the far key reads zero
+    L.check(lib.pi_op_channel_recurrence(DELTA, devs[0].ptr, D, devs[1].ptr, D, devs[2].ptr, V, devs[3].ptr, D, 0, None, None, devs[4].ptr, 1, None, 1, 1.0, 1, 1, D, V, sd.ptr, devs[5].ptr, T, 1, od.ptr, V, None))
+    assert np.abs(od.get(np.float32, (T, V))).max() < 1e-6
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("heads,n,per_head,act", [(3, 5, 0, SIGMOID), (2, 70, 1, NONE), (5, 130, 1, SILU), (1, 1, 0, NONE)])
+def test_head_norm_weight_gate(heads, n, per_head, act):
+    U, lib = gpu()
+    rng = np.random.default_rng(n)
+    T = 4
+    y, gate = (rng.standard_normal((T, heads * n + 2)) * 3).astype(np.float32), rng.standard_normal((T, heads * n + 1)).astype(np.float32)
+    w = rng.standard_normal(heads * n if per_head else n).astype(np.float32)
+    yd, gd, wd, od = U.Dev(y), U.Dev(gate), U.Dev(w), U.Dev(nbytes=4 * T * heads * n)
+    L.check(lib.pi_op_head_norm_gate(yd.ptr, heads * n + 2, heads, n, wd.ptr, per_head, gd.ptr, heads * n + 1, act, 1e-4, T, od.ptr, heads * n, None))
+    want = np.zeros((T, heads, n))
+    for t in range(T):
+        for h in range(heads):
+            g = gate[t, h * n:(h + 1) * n].astype(np.float64)
+            g = O.sigmoid(g) if act == SIGMOID else O.silu(g) if act == SILU else g
+            want[t, h] = O.unit_rms(y[t, h * n:(h + 1) * n].astype(np.float64), 1e-4) * (w[h * n:(h + 1) * n] if per_head else w) * g
+    assert rel_rms(od.get(np.float32, (T, heads, n)), want) < 3e-6
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D,V,R", [(3, 1, 8, 6, 4), (4, 4, 70, 66, 70), (2, 1, 5, 130, 0), (6, 2, 88, 10, 44)])
+def test_queries_and_keys_rotated_in_neighbour_pairs_then_normed(H, G, D, V, R):
+    U, lib = gpu()
+    rng = np.random.default_rng(D + V)
+    T, n_ctx, first, stride = 5, 20, 9, H * D + G * (D + V) + 3
+    buf = rng.standard_normal((T, stride)).astype(np.float32)
+    pos = np.array([0, 1, 37, 38, 399], np.int32)
+    tab = lib.pi_rotary_table_create(400, R, 777.0)
+    bd, pd, dyn = U.Dev(buf), U.Dev(pos), U.Dev(np.array([first, first + T, T, 0], np.int32))
+    qo, kc, vc, cp = U.Dev(nbytes=4 * T * H * D), U.Dev(np.zeros((n_ctx, G * D), np.float32)), U.Dev(np.zeros((n_ctx, G * V), np.float32)), U.Dev(np.full(n_ctx, -1, np.int32))
+    L.check(lib.pi_op_qkv_prepare_ex(bd.ptr, bd.ptr + 4 * H * D, bd.ptr + 4 * (H * D + G * D), stride, None, None, 1e-4, H, G, D, V, tab, 0, 1, 0, pd.ptr, T, qo.ptr, H * D, kc.ptr, vc.ptr, cp.ptr, dyn.ptr, None))
+    q, k, v, cpos = qo.get(np.float32, (T, H, D)), kc.get(np.float32, (n_ctx, G, D)), vc.get(np.float32, (n_ctx, G, V)), cp.get(np.int32, (n_ctx,))
+    b64 = buf.astype(np.float64)
+    for t in range(T):
+        for h in range(H):
+            assert rel_rms(q[t, h], O.unit_rms(O.rotate_pairs(b64[t, h * D:(h + 1) * D], int(pos[t]), R, 777.0), 1e-4)) < 3e-6
+        for g in range(G):
+            assert rel_rms(k[first + t, g], O.unit_rms(O.rotate_pairs(b64[t, H * D + g * D:H * D + (g + 1) * D], int(pos[t]), R, 777.0), 1e-4)) < 3e-6
+            o = H * D + G * D + g * V
+            assert np.array_equal(v[first + t, g], buf[t, o:o + V])                                # values are cached as they are
+    assert list(cpos[first:first + T]) == list(pos) and (cpos[:first] == -1).all() and (cpos[first + T:] == -1).all()
+    lib.pi_rotary_table_free(tab)
+
+
+def softmax_attention_ref(q, kc, vc, cpos, vis, pos, scale, cap, chunk, sink, H, G):
+    T, V = q.shape[0], vc.shape[2]
+    out = np.zeros((T, H, V))
+    for t in range(T):
+        for h in range(H):
+            g = h // (H // G)
+            cells = [c for c in range(kc.shape[0]) if vis[t, c] and not (chunk and cpos[c] // chunk != pos[t] // chunk)]
+            s = np.array([q[t, h].astype(np.float64) @ kc[c, g] for c in cells]) * scale
+            if cap:
+                s = cap * np.tanh(s / cap)
+            e = np.exp(s - s.max()) if len(cells) else np.zeros(0)
+            den = e.sum() + (np.exp(-s.max()) if sink and len(cells) else 0.0)
+            for w, c in zip(e / den if len(cells) else [], cells):
+                out[t, h] += w * vc[c, g]
+    return out
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D,V,chunk,n_kv,T", [(1, 1, 4, 6, 3, 20, 2), (3, 1, 8, 6, 7, 70, 5), (8, 2, 80, 72, 48, 700, 9), (4, 4, 33, 130, 100, 300, 4), (12, 2, 16, 24, 0, 520, 3), (2, 2, 64, 64, 512, 1100, 2)])
+@pytest.mark.parametrize("sink", [True, False])
+def test_softmax_attention_in_chunks_against_explicit_sums(H, G, D, V, chunk, n_kv, T, sink):
+    """cells in any order, garbage behind the live cells and in another sequence's cells, large scores (the running maximum matters), with and without the sink and the cap"""
+    U, lib = gpu()
+    rng = np.random.default_rng(H + D + n_kv)
+    n_ctx = n_kv + 13
+    kc, vc = (rng.standard_normal((n_ctx, G, D)) * 1.5).astype(np.float32), rng.standard_normal((n_ctx, G, V)).astype(np.float32)
+    kc[n_kv:], vc[n_kv:] = np.nan, np.nan
+    cpos = rng.permutation(n_ctx).astype(np.int32)
+    pos = np.sort(rng.integers(n_kv // 2, n_kv, T)).astype(np.int32)
+    vis = (cpos[None, :n_kv] <= pos[:, None]) & (rng.random((T, n_kv)) < 0.8)
+    for t in range(T):
+        vis[t, rng.integers(0, n_kv)] = True
+    q = (rng.standard_normal((T, H, D)) * 2).astype(np.float32)
+    cap = 9.0 if H % 2 else 0.0
+    qd, kd, vd, cd, md, pd = U.Dev(q), U.Dev(kc), U.Dev(vc), U.Dev(cpos), U.Dev(pack_mask(vis, n_kv)), U.Dev(pos)
+    od, dyn = U.Dev(nbytes=4 * T * H * V), U.Dev(np.array([0, n_kv, T, 0], np.int32))
+    L.check(lib.pi_op_chunk_attention_ex(qd.ptr, H * D, kd.ptr, vd.ptr, cd.ptr, md.ptr, pd.ptr, None, None, 0, NONE, 0.6, 1.0, 2 if sink else 1, cap, chunk, H, G, D, V, T, n_kv, od.ptr, H * V, dyn.ptr, None))
+    want = softmax_attention_ref(q, kc[:n_kv].astype(np.float64), vc[:n_kv].astype(np.float64), cpos, vis, pos, 0.6, cap, chunk, sink, H, G)
+    assert rel_rms(od.get(np.float32, (T, H, V)), want) < 5e-6
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("chunk,p", [(8, 23), (8, 24), (64, 127), (64, 128), (5, 4), (200, 399), (200, 400)])
+def test_chunk_border_keys_and_the_sink(chunk, p):
+    """one key on the chunk's first position that must take (nearly) all the mass, one just before it with a far larger score that must not count; a token alone with a sink keeps half"""
+    U, lib = gpu()
+    D, V, n_kv = 4, 3, p + 1
+    kc, vc = np.zeros((n_kv, 1, D), np.float32), np.zeros((n_kv, 1, V), np.float32)
+    start = p // chunk * chunk
+    kc[start, 0, 0], vc[start, 0] = 12.0, [1.0, 2.0, 3.0]
+    if start > 0:
+        kc[start - 1, 0, 0], vc[start - 1, 0] = 40.0, [100.0, 100.0, 100.0]
+    q = np.zeros((1, 1, D), np.float32)
+    q[0, 0, 0] = 1.0
+    cpos, vis = np.arange(n_kv, dtype=np.int32), np.ones((1, n_kv), bool)
+    devs = [U.Dev(a) for a in (q, kc, vc, cpos, pack_mask(vis, n_kv), np.array([p], np.int32), np.array([0, n_kv, 1, 0], np.int32))]
+    od = U.Dev(nbytes=4 * V)
+    L.check(lib.pi_op_chunk_attention_ex(devs[0].ptr, D, devs[1].ptr, devs[2].ptr, devs[3].ptr, devs[4].ptr, devs[5].ptr, None, None, 0, NONE, 1.0, 1.0, 2, 0.0, chunk, 1, 1, D, V, 1, n_kv, od.ptr, V, devs[6].ptr, None))
+    n_in = p - start + 1
+    want = np.exp(12.0) / (1.0 + np.exp(12.0) + (n_in - 1)) * np.array([1.0, 2.0, 3.0])
+    assert np.allclose(od.get(np.float32, (V,)), want, rtol=1e-5)
+    devs[5] = U.Dev(np.array([start], np.int32))                       # the chunk's first token sees itself and the sink
+    devs[4] = U.Dev(pack_mask(cpos[None, :] <= start, n_kv))
+    L.check(lib.pi_op_chunk_attention_ex(devs[0].ptr, D, devs[1].ptr, devs[2].ptr, devs[3].ptr, devs[4].ptr, devs[5].ptr, None, None, 0, NONE, 0.0, 1.0, 2, 0.0, chunk, 1, 1, D, V, 1, n_kv, od.ptr, V, devs[6].ptr, None))
+    assert np.allclose(od.get(np.float32, (V,)), 0.5 * np.array([1.0, 2.0, 3.0]), rtol=1e-6)
+
+
+# ---- whole models through llama_decode ---------------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("variant", list(VARIANTS))
+@pytest.mark.parametrize("exact", [True, False])
+def test_prompt_portions_and_decoding_agree_with_the_oracle(tmp_path, variant, exact):
+    m = small_model(seed=11, layers=VARIANTS[variant], width=64 if variant == "wide_heads" else 40)
+    rng = np.random.default_rng(5)
+    toks = [int(t) for t in rng.integers(0, VOCAB, 75)]
+    want = O.run(m, toks)
+    e = Engine(tmp_path, m, n_ctx=96, n_batch=48, exact=exact)
+    tol = TOL[exact] * (3 if variant == "wide_heads" else 1)
+    whole = np.concatenate([e.ctx.feed(toks[:48], 0, 0), e.ctx.feed(toks[48:], 48, 0)])
+    assert logit_err(whole, want).max() < tol
+    e.ctx.seq_rm(0, -1, -1)
+    parts, at = [], 0
+    for n in [2, 3, 31, 2, 1, 1, 7, 2, 5, 1, 1, 1, 2, 16]:                 # portions down to two tokens and single tokens, cut inside chunks and convolution windows
+        parts.append(e.ctx.feed(toks[at:at + n], at, 1))
+        at += n
+    assert at == 75 and logit_err(np.concatenate(parts), want).max() < tol
+    e.ctx.seq_rm(1, -1, -1)
+    single = np.concatenate([e.ctx.feed(toks[i:i + 1], i, 2) for i in range(40)])
+    assert logit_err(single, want[:40]).max() < tol
+    e.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("exact", [True, False])
+def test_a_wider_model_with_long_passes(tmp_path, exact):
+    """widths and passes that reach the matrix-core products and the tiles of the recurrences: 300 tokens in passes of 128, then single tokens"""
+    layers = [O.delta_layer(heads=4, kv_heads=2, dim=32, vdim=48, conv=4, decay_rank=8, gate_rank=8, mlp=None),
+              O.parallel_layer(heads=4, kv_heads=2, dim=64, vdim=32, chunk=100, rot_dims=16, scale=0.2, r_heads=4, r_dim=32, decay_rank=8, mlp=O.dense_mlp(256))]
+    m = small_model(seed=13, layers=layers, width=128, vocab=200)
+    rng = np.random.default_rng(6)
+    toks = [int(t) for t in rng.integers(0, 200, 320)]
+    want = O.run(m, toks)
+    e = Engine(tmp_path, m, n_ctx=330, n_batch=128, exact=exact)
+    got = np.concatenate([e.ctx.feed(toks[:300], 0, 0)] + [e.ctx.feed(toks[i:i + 1], i, 0) for i in range(300, 320)])
+    assert logit_err(got, want).max() < TOL[exact] * 2
+    e.close()
+
+
+@pytest.mark.gpu
+def test_residual_stream_layer_by_layer(tmp_path):
+    """models cut after 1, 2, ... layers give the oracle's logits, so the first wrong layer would be named"""
+    full = small_model(seed=4)
+    toks = [5, 17, 3, 80, 0, 41, 41, 7, 9, 9, 30]
+    for n in range(1, 5):
+        m = {"config": dict(full["config"], layers=full["config"]["layers"][:n]), "tensors": full["tensors"]}
+        e = Engine(tmp_path, m, n_ctx=32, n_batch=8, name="cut%d" % n)
+        assert logit_err(e.ctx.feed(toks, 0, 0), O.run(m, toks)).max() < TOL[True], n
+        e.close()
+
+
+@pytest.mark.gpu
+def test_first_tokens_and_the_pair_table(tmp_path):
+    """a sequence's first token takes the table's last row whatever was fed before in its slot; later tokens take the row of (previous, current) across passes"""
+    m = small_model(seed=17)
+    e = Engine(tmp_path, m, n_ctx=64, n_batch=8, slots=1)
+    for toks in ([7], [7, 7], [80, 7, 3], [3, 80, 7, 7, 2, 2, 2, 9, 1, 4, 4]):
+        got = np.concatenate([e.ctx.feed(toks[i:i + 3], i, 0) for i in range(0, len(toks), 3)])
+        assert logit_err(got, O.run(m, toks)).max() < TOL[True], toks
+        e.ctx.seq_rm(0, -1, -1)
+    e.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("exact", [True, False])
+def test_batches_of_unequal_requests_equal_each_alone(tmp_path, exact):
+    m = small_model(seed=21)
+    rng = np.random.default_rng(8)
+    reqs = [[int(t) for t in rng.integers(0, VOCAB, n)] for n in (23, 5, 14)]
+    want = [O.run(m, r) for r in reqs]
+    e = Engine(tmp_path, m, n_ctx=128, n_batch=64, exact=exact)
+    first = [9, 2, 14]
+    toks = sum((r[:n] for r, n in zip(reqs, first)), [])
+    pos = sum((list(range(n)) for n in first), [])
+    seqs = sum(([[s]] * n for s, n in enumerate(first)), [])
+    lg = e.ctx.decode(toks, pos, seqs)
+    at, errs = 0, []
+    for s, n in enumerate(first):
+        errs.append(logit_err(lg[at:at + n], want[s][:n]))
+        at += n
+    extra = [int(t) for t in rng.integers(0, VOCAB, 6)]
+    toks = reqs[1][2:] + extra + reqs[0][9:]
+    pos = list(range(2, 5)) + list(range(6)) + list(range(9, 23))
+    seqs = [[1]] * 3 + [[3]] * 6 + [[0]] * 14
+    lg = e.ctx.decode(toks, pos, seqs)
+    errs += [logit_err(lg[:3], want[1][2:]), logit_err(lg[3:9], O.run(m, extra)), logit_err(lg[9:], want[0][9:])]
+    assert np.concatenate(errs).max() < TOL[exact], [float(x.max()) for x in errs]
+    e.close()
+
+
+@pytest.mark.gpu
+def test_freed_cells_and_slots_are_used_again(tmp_path):
+    """more requests than slots and cells, one after the other and interleaved: a finished request gives back what it held, the next one starts from nothing (no key, no
+    convolution input, no shifted token, no previous token, no state of the earlier owner)"""
+    m = small_model(seed=31)
+    rng = np.random.default_rng(9)
+    e = Engine(tmp_path, m, n_ctx=48, n_batch=16, slots=2)
+    for round_ in range(5):
+        a = [int(t) for t in rng.integers(0, VOCAB, 20 + round_)]
+        b = [int(t) for t in rng.integers(0, VOCAB, 11)]
+        la = e.ctx.feed(a[:7], 0, 0)
+        lb = e.ctx.feed(b, 0, 1)
+        la = np.concatenate([la, e.ctx.feed(a[7:], 7, 0)])
+        assert e.ctx.state_slots_used() == 2
+        with pytest.raises(L.PipeInferError):
+            e.ctx.decode([1], [0], [[2]])
+        e.ctx.seq_rm(1, -1, -1)
+        lc = e.ctx.feed(b[:5], 0, 2)
+        for got, toks in ((la, a), (lb, b), (lc, b[:5])):
+            assert logit_err(got, O.run(m, toks)).max() < TOL[True], round_
+        e.ctx.seq_rm(0, -1, -1)
+        e.ctx.seq_rm(2, -1, -1)
+        assert e.ctx.state_slots_used() == 0
+    a = [int(t) for t in rng.integers(0, VOCAB, 12)]
+    e.ctx.feed(a[:8], 0, 0)
+    e.ctx.seq_cp(0, 1, -1, -1)                                      # a copy of a sequence (cells shared; states, convolution inputs, shifted and previous token copied) continues like the original
+    assert logit_err(e.ctx.feed(a[8:] + [50, 51], 8, 1), O.run(m, a + [50, 51])[8:]).max() < TOL[True]
+    assert logit_err(e.ctx.feed(a[8:] + [60], 8, 0), O.run(m, a + [60])[8:]).max() < TOL[True]
+    e.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("exact", [True, False])
+def test_chunk_borders_show_in_prompts_and_in_decoding(tmp_path, exact):
+    """sharp attention (a large score scale, no cap worth the name) over several hundred tokens, chunk sizes that are no divisors of the pass width: a key that is wrongly seen or lost
+    at a chunk's border, or a state that forgets, shows far above rounding — the same model with chunks one position longer is far away"""
+    layers = [O.parallel_layer(heads=2, kv_heads=1, dim=8, vdim=8, chunk=50, rot_dims=4, scale=2.5, softcap=30.0, r_heads=2, r_dim=4, mlp=None),
+              O.delta_layer(mlp=None),
+              O.parallel_layer(heads=3, kv_heads=3, dim=4, vdim=6, chunk=37, rot_dims=2, scale=3.0, softcap=None, mlp=O.dense_mlp(16))]
+    m = small_model(seed=41, layers=layers, width=32)
+    rng = np.random.default_rng(12)
+    toks = [int(t) for t in rng.integers(0, VOCAB, 330)]
+    want = O.run(m, toks)
+    e = Engine(tmp_path, m, n_ctx=340, n_batch=128, exact=exact)
+    got = np.concatenate([e.ctx.feed(toks[:290], 0, 0)] + [e.ctx.feed(toks[i:i + 1], i, 0) for i in range(290, 330)])       # decoding passes positions 296 and 300: a border of each layer
+    err = logit_err(got, want)
+    assert err.max() < TOL[exact]
+    longer = json.loads(json.dumps(m["config"]))
+    longer["layers"][0]["mixer"]["left"]["mask"]["size"] = 51
+    off = logit_err(got, O.run({"config": longer, "tensors": m["tensors"]}, toks))
+    assert off[[50, 100, 299, 300]].min() > (100 if exact else 2) * TOL[exact]                    # (a chunk that is one position off would be seen, in the prompt and among the decoded tokens)
+    e.close()
+
+
+@pytest.mark.gpu
+def test_long_decoding_token_by_token(tmp_path):
+    m = small_model(seed=45)
+    rng = np.random.default_rng(13)
+    toks = [int(t) for t in rng.integers(0, VOCAB, 200)]
+    want = O.run(m, toks)
+    e = Engine(tmp_path, m, n_ctx=224, n_batch=8, exact=True)
+    got = np.concatenate([e.ctx.feed(toks[:3], 0, 0)] + [e.ctx.feed(toks[i:i + 1], i, 0) for i in range(3, 200)])
+    assert logit_err(got, want).max() < TOL[True]
+    e.close()
+
+
+@pytest.mark.gpu
+def test_greedy_generation_through_the_engine(tmp_path):
+    m = small_model(seed=51)
+    prompt = [3, 14, 15, 72, 65, 35]
+    e = Engine(tmp_path, m, n_ctx=160, n_batch=16, exact=True)
+    got = e.ctx.generate(prompt, 100)
+    want = O.greedy(m, prompt, 100)
+    k = next((i for i, (a, b) in enumerate(zip(got, want)) if a != b), len(want))
+    if k < len(want):                                               # (an arg-max between two nearly equal logits may fall either way in fp32 against float64: it must be a near tie)
+        lg = O.run(m, prompt + want[:k])[-1]
+        assert abs(lg[got[k]] - lg[want[k]]) < 1e-3 * np.abs(lg).max()
+    assert k >= 20
+    e.close()
+
+
+@pytest.mark.gpu
+def test_graph_replays_equal_eager_launches(tmp_path):
+    m = small_model(seed=61)
+    rng = np.random.default_rng(3)
+    toks = [int(t) for t in rng.integers(0, VOCAB, 60)]
+    outs = []
+    for graphs in (True, False):
+        e = Engine(tmp_path, m, n_ctx=64, n_batch=16, exact=False, name="g%d" % graphs)
+        e.ctx.set_graphs(graphs)
+        lg = []
+        for rep in range(3):
+            lg.append(np.concatenate([e.ctx.feed(toks[:37], 0, rep % 2), e.ctx.feed(toks[37:38], 37, rep % 2), e.ctx.feed(toks[38:], 38, rep % 2)]))
+            e.ctx.seq_rm(rep % 2, -1, -1)
+        assert all(np.array_equal(lg[0], x) for x in lg[1:])
+        outs.append(lg[0])
+        e.close()
+    assert np.array_equal(outs[0], outs[1])
+
+
+@pytest.mark.gpu
+def test_generate_command_line(tmp_path, capsys):
+    from pipeinfer_amd.tools import generate as G
+    m = small_model(seed=71)
+    folder = str(tmp_path / "g")
+    write(folder, m)
+    assert G.main(["--model", folder, "--prompt-ids", "5,6,7", "--n-predict", "12", "--float32"]) == 0
+    greedy = [int(t) for t in capsys.readouterr().out.strip().split(",")]
+    want = O.greedy(m, [5, 6, 7], 12)
+    k = next((i for i, (a, b) in enumerate(zip(greedy, want)) if a != b), 12)
+    assert k >= 6
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_trace_runner_replays_steps_and_writes_the_wanted_rows(tmp_path, dtype):
+    import subprocess
+    import sys
+    m = small_model(seed=81, layers=VARIANTS["edges"])
+    folder, out = str(tmp_path / "model"), str(tmp_path / "out")
+    write(folder, m)
+    rng = np.random.default_rng(5)
+    a, b = [int(t) for t in rng.integers(0, VOCAB, 41)], [int(t) for t in rng.integers(0, VOCAB, 9)]
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:3], "want": [0, 2]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[3:33], "want": []}], "end": []},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[33:40], "want": [6, 1]}], "end": []},
+             {"step": 3, "entries": [{"id": "a", "tokens": a[40:], "want": [0]}], "end": ["a"]},
+             {"step": 4, "entries": [{"id": "b", "tokens": b, "want": [8]}], "end": ["b"]}]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dtype, "--out", out, "--max-tokens", "48", "--n-batch", "16"],
+                       input="".join(json.dumps(x) + "\n" for x in steps), capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done")] == ["done %d" % i for i in range(5)]
+    la, lb = O.run(m, a), O.run(m, b)
+    want = {0: la[[0, 2]], 2: la[[39, 34]], 3: la[[40]], 4: lb[[8]]}
+    assert sorted(os.listdir(out)) == sorted("%d.f32" % k for k in want)
+    for k, w in want.items():
+        got = np.fromfile(os.path.join(out, "%d.f32" % k), "<f4").reshape(-1, VOCAB)
+        assert got.shape == w.shape and logit_err(got, w).max() < TOL[dtype == "float32"], k
