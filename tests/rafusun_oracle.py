@@ -232,48 +232,48 @@ def random_model(rng, vocab, width, layers, eps=1e-5, alpha=1.7, embed_scale=3.0
     def near_one(n):
         return bf16_round((1.0 + 0.3 * rng.standard_normal(n)).astype(np.float32)).astype(np.float64)
 
-    T = {"embed": w(vocab, width, s=0.5), "bigram": w(buckets + 1, width, s=1.0), "head": w(vocab, width), "final.norm": near_one(width)}
+    T = {"embed": w(vocab, width, s=0.4), "bigram": w(buckets + 1, width, s=0.8), "head": w(vocab, width), "final.norm": near_one(width)}
     cfg_layers = []
     for i, L in enumerate(layers):
         p = "l%d." % i
         L = dict(L)
         ranks = L.pop("_ranks")
         cfg_layers.append(L)
-        T[p + "norm1"], T[p + "ls1"] = near_one(width), rb(w(width, s=1.0) + 1.0)
+        T[p + "norm1"], T[p + "ls1"] = near_one(width), rb(w(width, s=0.5) + 1.0)
         mx, m = L["mixer"], p + "mix."
         if L["type"] == "channel_delta":
             H, G, D, V, taps = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"], mx["conv"]
             for n, rows in (("q", G * D), ("k", G * D), ("v", H * V)):
-                T[m + n] = w(rows, width, s=1.0)
+                T[m + n] = w(rows, width)
                 T[m + n + ".conv"] = w(rows, taps, s=0.7)
-            T[m + "b"] = w(H, width, s=1.0)
+            T[m + "b"] = w(H, width)
             T[m + "A_log"] = w(H, s=0.5)
             T[m + "dt_bias"] = rb(w(H * D, s=1.0) - 1.0)
-            T[m + "a1"], T[m + "a2"] = w(ranks[0], width, s=1.0), w(H * D, ranks[0])
-            T[m + "g1"], T[m + "g2"] = w(ranks[1], width, s=1.0), w(H * V, ranks[1])
+            T[m + "a1"], T[m + "a2"] = w(ranks[0], width), w(H * D, ranks[0])
+            T[m + "g1"], T[m + "g2"] = w(ranks[1], width), w(H * V, ranks[1])
             T[m + "norm"] = near_one(V)
-            T[m + "o"] = w(width, H * V, s=1.0)
+            T[m + "o"] = w(width, H * V)
         else:
             A, R = mx["left"], mx["right"]
-            T[m + "left.q"] = w(A["heads"] * A["dim"], width, s=1.0)
-            T[m + "left.k"] = w(A["kv_heads"] * A["dim"], width, s=1.0)
-            T[m + "left.v"] = w(A["kv_heads"] * A["vdim"], width, s=1.0)
-            T[m + "left.o"] = w(width, A["heads"] * A["vdim"], s=1.0)
+            T[m + "left.q"] = w(A["heads"] * A["dim"], width)
+            T[m + "left.k"] = w(A["kv_heads"] * A["dim"], width)
+            T[m + "left.v"] = w(A["kv_heads"] * A["vdim"], width)
+            T[m + "left.o"] = w(width, A["heads"] * A["vdim"])
             T[m + "left.out"], T[m + "right.out"] = near_one(width), near_one(width)
             inner = R["heads"] * R["dim"]
             for n in "rkvgw":
                 T[m + "right.mu." + n] = bf16_round(rng.uniform(0.0, 1.0, width).astype(np.float32)).astype(np.float64)
             for n in "rkvg":
-                T[m + "right." + n] = w(inner, width, s=1.0)
-            T[m + "right.w1"], T[m + "right.w2"] = w(ranks[0], width, s=1.0), w(inner, ranks[0], s=1.0)
+                T[m + "right." + n] = w(inner, width)
+            T[m + "right.w1"], T[m + "right.w2"] = w(ranks[0], width), w(inner, ranks[0])
             T[m + "right.w0"] = rb(w(inner, s=1.0) - 1.5)
             T[m + "right.u"] = w(R["heads"], R["dim"], s=0.7)
             T[m + "right.norm"] = near_one(inner)
-            T[m + "right.o"] = w(width, inner, s=1.0)
+            T[m + "right.o"] = w(width, inner)
         if L.get("mlp"):
             ff = L["mlp"]["ff"]
-            T[p + "norm2"], T[p + "ls2"] = near_one(width), rb(w(width, s=1.0) + 1.0)
-            T[p + "mlp.gate"], T[p + "mlp.up"], T[p + "mlp.down"] = w(ff, width, s=1.0), w(ff, width, s=1.0), w(width, ff, s=1.0)
+            T[p + "norm2"], T[p + "ls2"] = near_one(width), rb(w(width, s=0.5) + 1.0)
+            T[p + "mlp.gate"], T[p + "mlp.up"], T[p + "mlp.down"] = w(ff, width), w(ff, width), w(width, ff)
     config = {"architecture": "Rafusun", "vocab": vocab, "width": width, "norm": {"eps": eps}, "postln_alpha": alpha,
               "embedding": {"scale": embed_scale, "bigram": {"buckets": buckets, "mul_prev": mul_prev, "mul_cur": mul_cur}}, "layers": cfg_layers}
     return {"config": config, "tensors": T}
