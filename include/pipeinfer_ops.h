@@ -294,7 +294,10 @@ PI_API int pi_op_token_shift(const float * h_dev, int64_t h_stride, int n, const
 enum pi_recurrence_rule { PI_RULE_DELTA = 0, PI_RULE_BONUS = 1 };
 PI_API int pi_op_channel_recurrence(int rule, const float * q_dev, int64_t q_stride, const float * k_dev, int64_t k_stride, const float * v_dev, int64_t v_stride, const float * decay_raw_dev, int64_t decay_stride,
                                     int decay_mode, const float * decay_bias_dev, const float * a_log_dev, const float * beta_raw_dev, int64_t beta_stride, const float * bonus_dev, int qk_unit, float q_mult,
-                                    int heads, int qk_heads, int dim, int vdim, float * state_dev, const int32_t * rec_dev, int n_tok, int max_segments, float * out_dev, int64_t out_stride, void * stream);
+                                    int heads, int qk_heads, int dim, int vdim, float * state_dev, const int32_t * rec_dev, int n_tok, int max_segments, float * scratch_dev, size_t scratch_floats,
+                                    float * out_dev, int64_t out_stride, void * stream);
+/* passes of more than 32 tokens cut the sequences into pieces that run side by side (a column's step is affine in the column): floats of scratch they need; with less the pass is walked token by token */
+PI_API size_t pi_op_channel_recurrence_scratch_floats(int heads, int dim, int vdim, int n_tok, int max_segments);
 PI_API int pi_op_channel_recurrence_reserve(void);                 /* once per process, outside graph capture: the LDS limit wide keys need */
 /* out[t][h][i] = y[t][h][i] / sqrt(mean_i(y[t][h]^2) + eps) * w[(w_per_head ? h * n : 0) + i] * act(gate[t][h][i]) (gate nullable; gate_act PI_ACT_NONE, _SIGMOID or _SILU); out may be y */
 PI_API int pi_op_head_norm_gate(const float * y_dev, int64_t y_stride, int heads, int n, const float * w_dev, int w_per_head, const float * gate_dev, int64_t gate_stride, int gate_act, float eps, int n_tok,

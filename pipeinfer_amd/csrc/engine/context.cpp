@@ -114,11 +114,13 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
                 const pi_channel_delta & D = H.delta;
                 in_w = std::max(in_w, (size_t) D.in_rows());
                 att_w = std::max(att_w, (size_t) D.channels() + (size_t) D.heads * D.dim + (size_t) 2 * D.heads * D.vdim);
+                ctx->rec_scratch_floats = std::max(ctx->rec_scratch_floats, pi_op_channel_recurrence_scratch_floats(D.heads, D.dim, D.vdim, nb, ctx->slots->size()));
             } else {
                 const pi_gate_attention & A = H.left; const pi_time_mix & R = H.shift;
                 ctx->lat_off[i] = lat; lat += (size_t) ctx->n_ctx * H.cell_floats();
                 in_w = std::max(in_w, (size_t) A.in_rows() + (size_t) 5 * width);
                 att_w = std::max(att_w, (size_t) A.heads * (A.dim + A.vdim) + (size_t) 7 * R.inner() + (size_t) R.decay_rank);
+                ctx->rec_scratch_floats = std::max(ctx->rec_scratch_floats, pi_op_channel_recurrence_scratch_floats(R.heads, R.dim, R.dim, nb, ctx->slots->size()));
                 positions = true;
             }
             ctx->rec_off[i] = rec; rec += (size_t) ctx->slots->size() * H.state_floats();
@@ -443,7 +445,7 @@ static bool forward_post_norm_blocks(llama_context * ctx, int n_tok, int n_kv) {
             OP_OK(pi_op_dense(W.w_a2, P + ch, pw, n_tok, A2, hd, PI_ACT_NONE, hd, PI_ACT_NONE, ex, s));
             OP_OK(pi_op_dense(W.w_g2, P + ch + D.decay_rank, pw, n_tok, G2, hv, PI_ACT_NONE, hv, PI_ACT_NONE, ex, s));
             OP_OK(pi_op_channel_recurrence(PI_RULE_DELTA, C, ch, C + gd, ch, C + 2 * gd, ch, A2, hd, 2, W.dt_bias, W.a_log, P + ch + D.decay_rank + D.gate_rank, pw, nullptr, 1, 1.0f / sqrtf((float) D.dim), D.heads, D.kv_heads, D.dim, D.vdim,
-                                           S, ctx->rec_dev, n_tok, n_slots, O, hv, s));
+                                           S, ctx->rec_dev, n_tok, n_slots, ctx->rec_scratch, ctx->rec_scratch_floats, O, hv, s));
             trace(ctx, "rec", (int) il, O, hv, n_tok);
             OP_OK(pi_op_head_norm_gate(O, hv, D.heads, D.vdim, W.mix_norm, 0, G2, hv, PI_ACT_SIGMOID, eps, n_tok, O, hv, s));
             OP_OK(pi_op_dense(W.w_o, O, hv, n_tok, Y, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
@@ -470,7 +472,7 @@ static bool forward_post_norm_blocks(llama_context * ctx, int n_tok, int n_kv) {
             OP_OK(pi_op_dense(W.w_w1, M + 4 * width, mw, n_tok, W1, R.decay_rank, PI_ACT_TANH, R.decay_rank, PI_ACT_TANH, ex, s));
             OP_OK(pi_op_dense(W.w_w2, W1, R.decay_rank, n_tok, WD, inner, PI_ACT_NONE, inner, PI_ACT_NONE, ex, s));
             OP_OK(pi_op_channel_recurrence(PI_RULE_BONUS, RK, 4 * inner, RK + inner, 4 * inner, RK + 2 * inner, 4 * inner, WD, inner, 1, W.w0, nullptr, nullptr, 0, W.bonus, 0, 1.0f, R.heads, R.heads, R.dim, R.dim,
-                                           S, ctx->rec_dev, n_tok, n_slots, O2, inner, s));
+                                           S, ctx->rec_dev, n_tok, n_slots, ctx->rec_scratch, ctx->rec_scratch_floats, O2, inner, s));
             trace(ctx, "rec", (int) il, O2, inner, n_tok);
             OP_OK(pi_op_head_norm_gate(O2, inner, R.heads, R.dim, W.mix_norm, 1, RK + 3 * inner, 4 * inner, PI_ACT_NONE, eps, n_tok, O2, inner, s));
             OP_OK(pi_op_dense(W.w_o2, O2, inner, n_tok, Y2, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));

@@ -160,56 +160,89 @@ extern "C" int pi_op_token_shift(const float * h, int64_t h_stride, int n, const
 }
 
 // ---- recurrences with a decay per key channel ------------------------------------------------------------------------------------------------------------------
-// Workgroup (head, block of value columns, run of the pass): thread (column j, part sp of R) keeps S[i][j] for its DPT rows i in registers and walks the run's tokens in order; q, k,
+// Workgroup (head, block of value columns, piece of the pass): thread (column j, part sp of R) keeps S[i][j] for its DPT rows i in registers and walks the piece's tokens in order; q, k,
 // the decays and v of CR_TB tokens at a time are staged (and finished: decays formed, unit vectors, sigmoid) in LDS.  A value column never meets another: o_j, u_j and S[:, j]
 // depend on column j alone, so the only exchange is the sum over the R parts of a column (neighbouring lanes).
 //   delta:  S <- g S;  a = S^T k, c = S^T q (one pass over the registers);  u = beta (v - a);  o = c + u (k . q);  S <- S + k u
 //   bonus:  c = S^T q;  o = c + v (sum_i q_i b_i k_i);  S <- g S + k v
+// A pass of up to CR_TB tokens (or keys too wide for the scan's tile) is ONE launch, mode 0: a piece is a sequence's whole run, S comes from and goes back to HBM.  Longer passes cut
+// every run into pieces of CR_TB tokens that run side by side, because a column's step is affine in the column, s <- A_t s + b_t v_j with A_t the same for every column:
+//   mode 1  every piece but a run's last, with dim extra columns: L_p = the state the piece builds from ZERO, and T_p = A_n .. A_1, whose column c is what the piece makes of the unit
+//           vector e_c with v = 0 — the same walk over a column that starts as e_c — both into scratch [piece][head][dim][vdim + dim]
+//   k_channel_state_scan  per run, piece by piece: S_in(p + 1) = T_p S_in(p) + L_p, S_in(0) = the slot's state (or zero); scratch[p][..][0 .. vdim) <- S_in(p)
+//   mode 2  every piece from its true S_in(p): outputs; a run's last piece leaves the slot's new state
 #define CR_TB 32
 #define CR_MAXRUNS 256
+#define CR_SCAN_MAXDIM 128                        // widest key whose transition matrix the scan keeps in LDS
+// the pass's runs in order (a run: the consecutive tokens of one slot): every thread looks at its own tokens for a run's first one, the few found are ranked by position.  first[r] in `sorted`
+static __device__ __forceinline__ int cr_runs(const int32_t * __restrict__ rec, int n_tok, int * bnd, int * sorted, int * nb) {
+    if (threadIdx.x == 0) *nb = 0;
+    __syncthreads();
+    for (int t = threadIdx.x; t < n_tok; t += blockDim.x)
+        if (t == 0 || (rec[t] & ~CM_FRESH) != (rec[t - 1] & ~CM_FRESH)) { const int at = atomicAdd(nb, 1); if (at < CR_MAXRUNS) bnd[at] = t; }
+    __syncthreads();
+    const int n = min(*nb, CR_MAXRUNS);
+    for (int i = threadIdx.x; i < n; i += blockDim.x) {
+        int rank = 0;
+        for (int o = 0; o < n; o++) rank += bnd[o] < bnd[i];
+        sorted[rank] = bnd[i];
+    }
+    __syncthreads();
+    return n;
+}
 template <int DPT, int RULE>
 __global__ void __launch_bounds__(256) k_channel_recurrence(const float * __restrict__ q, int64_t qs, const float * __restrict__ k, int64_t ks, const float * __restrict__ v, int64_t vs,
                                                             const float * __restrict__ draw, int64_t ds, int decay_mode, const float * __restrict__ dbias, const float * __restrict__ a_log,
                                                             const float * __restrict__ braw, int64_t bs, const float * __restrict__ bonus, int qk_unit, float q_mult,
-                                                            int heads, int hpg, int dim, int vdim, int R, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok,
-                                                            float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
+                                                            int heads, int hpg, int dim, int vdim, int R, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, int mode,
+                                                            float * __restrict__ scratch, float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
     extern __shared__ float lds[];                // q [CR_TB][dim] | k [CR_TB][dim] | g [CR_TB][dim] | v [CR_TB][cols]
-    __shared__ int seg[4], bnd[CR_MAXRUNS], nbnd; // first token, length, slot word of this workgroup's run, first token of the next run
+    __shared__ int seg[4], bnd[CR_MAXRUNS], sorted[CR_MAXRUNS], nbnd;      // seg: first token, length, slot word of this workgroup's piece, whether it is its run's last
     __shared__ float beta_t[CR_TB], dot_t[CR_TB];
     const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
-    // run number blockIdx.z of the pass (a run: the consecutive tokens of one slot).  Every thread looks at its own tokens for a run's first one, the few found are ranked by position
-    if (tid == 0) { nbnd = 0; seg[0] = 0; seg[1] = 0; seg[2] = -1; seg[3] = n_tok; }
-    __syncthreads();
-    for (int t = tid; t < n_tok; t += blockDim.x)
-        if (t == 0 || (rec[t] & ~CM_FRESH) != (rec[t - 1] & ~CM_FRESH)) { const int at = atomicAdd(&nbnd, 1); if (at < CR_MAXRUNS) bnd[at] = t; }
-    __syncthreads();
-    const int n_runs = min(nbnd, CR_MAXRUNS);
-    for (int i = tid; i < n_runs; i += blockDim.x) {
-        int rank = 0;
-        for (int o = 0; o < n_runs; o++) rank += bnd[o] < bnd[i];
-        if (rank == (int) blockIdx.z) { seg[0] = bnd[i]; seg[2] = rec[bnd[i]]; }
-        if (rank == (int) blockIdx.z + 1) seg[3] = bnd[i];
+    const int n_runs = cr_runs(rec, n_tok, bnd, sorted, &nbnd);
+    if (tid == 0) {                               // piece number blockIdx.z of the pass (mode 0: pieces are whole runs)
+        const int lseg = mode ? CR_TB : 0, want = blockIdx.z;
+        int ord = 0;
+        seg[1] = 0; seg[2] = -1;
+        for (int r = 0; r < n_runs; r++) {
+            const int t = sorted[r], e = r + 1 < n_runs ? sorted[r + 1] : n_tok;
+            const int nsub = lseg > 0 ? (e - t + lseg - 1) / lseg : 1;
+            if (want < ord + nsub) {
+                const int pc = want - ord;
+                seg[0] = lseg > 0 ? t + pc * lseg : t; seg[1] = lseg > 0 ? min(lseg, e - seg[0]) : e - t; seg[2] = rec[t]; seg[3] = pc == nsub - 1;
+                break;
+            }
+            ord += nsub;
+        }
     }
     __syncthreads();
-    if (tid == 0 && seg[2] >= 0) seg[1] = seg[3] - seg[0];
-    __syncthreads();
-    const int first = seg[0], len = seg[1], word = seg[2];
-    if (len == 0 || word < 0) return;
+    const int first = seg[0], len = seg[1], word = seg[2], last = seg[3];
+    if (len == 0 || word < 0 || (mode == 1 && last)) return;
     const int slot = word & ~CM_FRESH;
     const int cols = blockDim.x / R;
+    const int ncol = mode == 1 ? vdim + dim : vdim, sw = vdim + dim;   // columns this launch walks; row stride of a piece's block in scratch
     const int j = blockIdx.y * cols + tid / R, sp = tid % R;
-    const bool col_ok = j < vdim;
+    const bool col_ok = j < ncol;
     const int hq = h / hpg;                                            // the q / k head this head reads
     float * S_hbm = state + ((int64_t) slot * heads + h) * dim * vdim;
+    float * S_scr = scratch ? scratch + ((int64_t) blockIdx.z * heads + h) * dim * sw : nullptr;
     float S[DPT];
 #pragma unroll
     for (int ii = 0; ii < DPT; ii++) {
         const int i = sp * DPT + ii;
-        S[ii] = (col_ok && i < dim && !(word & CM_FRESH)) ? S_hbm[(int64_t) i * vdim + j] : 0.0f;
+        float s0 = 0.0f;
+        if (col_ok && i < dim) {
+            if (mode == 1) s0 = j >= vdim && i == j - vdim ? 1.0f : 0.0f;
+            else if (mode == 2) s0 = S_scr[(int64_t) i * sw + j];
+            else if (!(word & CM_FRESH)) s0 = S_hbm[(int64_t) i * vdim + j];
+        }
+        S[ii] = s0;
     }
     float * qt = lds, * kt = qt + CR_TB * dim, * gt = kt + CR_TB * dim, * vt = gt + CR_TB * dim;
     const float ah = decay_mode == 2 ? expf(a_log[h]) : 0.0f;
+    const bool dim4 = (dim & 3) == 0;
     for (int t0 = 0; t0 < len; t0 += CR_TB) {
         const int nt = min(CR_TB, len - t0);
         __syncthreads();
@@ -226,7 +259,7 @@ __global__ void __launch_bounds__(256) k_channel_recurrence(const float * __rest
         if (tid < nt) beta_t[tid] = braw ? cm_sigmoid(braw[(int64_t) (first + t0 + tid) * bs + h]) : 1.0f;
         for (int idx = tid; idx < nt * cols; idx += blockDim.x) {
             const int tt = idx / cols, jj = blockIdx.y * cols + idx % cols;
-            vt[idx] = jj < vdim ? v[(int64_t) (first + t0 + tt) * vs + (int64_t) h * vdim + jj] : 0.0f;
+            vt[idx] = jj < vdim ? v[(int64_t) (first + t0 + tt) * vs + (int64_t) h * vdim + jj] : 0.0f;       // (the extra columns of mode 1 carry v = 0)
         }
         __syncthreads();
         for (int tt = wave; tt < nt; tt += nw) {                          // a wave per token: unit vectors, then the token's scalar (k . q, or sum q b k)
@@ -246,35 +279,112 @@ __global__ void __launch_bounds__(256) k_channel_recurrence(const float * __rest
         for (int tt = 0; tt < nt; tt++) {
             const float vj = vt[tt * cols + tid / R];
             const float * kr = kt + tt * dim + sp * DPT, * qr = qt + tt * dim + sp * DPT, * gr = gt + tt * dim + sp * DPT;
-            float a = 0.0f, c = 0.0f, o;
-            if (RULE == 0) {
+            float kk[DPT], a = 0.0f, c = 0.0f, o;
+            if (dim4) {                                                   // 16-byte LDS reads: a token costs 3 * DPT / 4 of them
 #pragma unroll
-                for (int ii = 0; ii < DPT; ii++)
-                    if (sp * DPT + ii < dim) { S[ii] *= gr[ii]; a = fmaf(S[ii], kr[ii], a); c = fmaf(S[ii], qr[ii], c); }
+                for (int ii = 0; ii < DPT; ii += 4) {
+                    if (sp * DPT + ii < dim) {
+                        const float4 kv = *(const float4 *) (kr + ii), qv = *(const float4 *) (qr + ii), gv = *(const float4 *) (gr + ii);
+                        kk[ii] = kv.x; kk[ii + 1] = kv.y; kk[ii + 2] = kv.z; kk[ii + 3] = kv.w;
+                        if (RULE == 0) {
+                            S[ii] *= gv.x; S[ii + 1] *= gv.y; S[ii + 2] *= gv.z; S[ii + 3] *= gv.w;
+                            a = fmaf(S[ii], kv.x, a); a = fmaf(S[ii + 1], kv.y, a); a = fmaf(S[ii + 2], kv.z, a); a = fmaf(S[ii + 3], kv.w, a);
+                        }
+                        c = fmaf(S[ii], qv.x, c); c = fmaf(S[ii + 1], qv.y, c); c = fmaf(S[ii + 2], qv.z, c); c = fmaf(S[ii + 3], qv.w, c);
+                        if (RULE == 1) { S[ii] *= gv.x; S[ii + 1] *= gv.y; S[ii + 2] *= gv.z; S[ii + 3] *= gv.w; }
+                    } else { kk[ii] = kk[ii + 1] = kk[ii + 2] = kk[ii + 3] = 0.0f; }
+                }
             } else {
 #pragma unroll
-                for (int ii = 0; ii < DPT; ii++)
-                    if (sp * DPT + ii < dim) c = fmaf(S[ii], qr[ii], c);
+                for (int ii = 0; ii < DPT; ii++) {
+                    if (sp * DPT + ii < dim) {
+                        kk[ii] = kr[ii];
+                        if (RULE == 0) { S[ii] *= gr[ii]; a = fmaf(S[ii], kk[ii], a); }
+                        c = fmaf(S[ii], qr[ii], c);
+                        if (RULE == 1) S[ii] *= gr[ii];
+                    } else kk[ii] = 0.0f;
+                }
             }
             if (R == 2) { if (RULE == 0) a += pi_partner<1>(a); c += pi_partner<1>(c); }
             else if (R == 4) { if (RULE == 0) { a += pi_partner<2>(a); a += pi_partner<1>(a); } c += pi_partner<2>(c); c += pi_partner<1>(c); }
             else for (int d = R >> 1; d > 0; d >>= 1) { if (RULE == 0) a += __shfl_xor(a, d, PI_WAVE); c += __shfl_xor(c, d, PI_WAVE); }
-            if (RULE == 0) {
-                const float u = beta_t[tt] * (vj - a);
-                o = fmaf(u, dot_t[tt], c);
+            const float u = RULE == 0 ? beta_t[tt] * (vj - a) : vj;       // what the token writes under its key
+            o = fmaf(u, dot_t[tt], c);
 #pragma unroll
-                for (int ii = 0; ii < DPT; ii++) if (sp * DPT + ii < dim) S[ii] = fmaf(kr[ii], u, S[ii]);
-            } else {
-                o = fmaf(vj, dot_t[tt], c);
-#pragma unroll
-                for (int ii = 0; ii < DPT; ii++) if (sp * DPT + ii < dim) S[ii] = fmaf(kr[ii], vj, gr[ii] * S[ii]);
-            }
-            if (col_ok && sp == 0) out[(int64_t) (first + t0 + tt) * os + (int64_t) h * vdim + j] = o;
+            for (int ii = 0; ii < DPT; ii++) S[ii] = fmaf(kk[ii], u, S[ii]);
+            if (mode != 1 && col_ok && sp == 0) out[(int64_t) (first + t0 + tt) * os + (int64_t) h * vdim + j] = o;
         }
     }
-    if (col_ok)
+    if (!col_ok) return;
+    if (mode == 1) {
+#pragma unroll
+        for (int ii = 0; ii < DPT; ii++) { const int i = sp * DPT + ii; if (i < dim) S_scr[(int64_t) i * sw + j] = S[ii]; }
+    } else if (last) {
 #pragma unroll
         for (int ii = 0; ii < DPT; ii++) { const int i = sp * DPT + ii; if (i < dim) S_hbm[(int64_t) i * vdim + j] = S[ii]; }
+    }
+}
+
+// grid (head, blocks of CR_SCAN_COLS value columns, run): per piece p of the run, in order: scratch[p] holds [L_p | T_p] coming in and S_in(p) (in L_p's place) going out.
+// A workgroup keeps its columns of S in LDS (two buffers) and T_p transposed ([c][i], so that a thread's rows are neighbours); thread (column j, row part): 8 rows at a time in registers.
+#define CR_SCAN_COLS 32
+__global__ void __launch_bounds__(256) k_channel_state_scan(int heads, int dim, int vdim, const float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, float * __restrict__ scratch,
+                                                            const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    extern __shared__ float lds[];                // T^T [dim][dim + 4] | S [2][dim][CR_SCAN_COLS]
+    __shared__ int seg[3], bnd[CR_MAXRUNS], sorted[CR_MAXRUNS], nbnd;      // slot word, first piece ordinal, pieces of the run (0: no such run)
+    const int tid = threadIdx.x, h = blockIdx.x, j0 = blockIdx.y * CR_SCAN_COLS;
+    const int n_runs = cr_runs(rec, n_tok, bnd, sorted, &nbnd);
+    if (tid == 0) {
+        int ord = 0;
+        seg[0] = -1; seg[2] = 0;
+        for (int r = 0; r < n_runs; r++) {
+            const int t = sorted[r], e = r + 1 < n_runs ? sorted[r + 1] : n_tok;
+            const int ns = (e - t + CR_TB - 1) / CR_TB;
+            if (r == (int) blockIdx.z) { seg[0] = rec[t]; seg[1] = ord; seg[2] = ns; break; }
+            ord += ns;
+        }
+    }
+    __syncthreads();
+    const int word = seg[0], sub0 = seg[1], nsub = seg[2];
+    if (nsub == 0 || word < 0) return;
+    const int slot = word & ~CM_FRESH, sw = vdim + dim, tp = dim + 4;
+    float * Tt = lds, * Sb = Tt + dim * tp;
+    const int jl = tid % CR_SCAN_COLS, part = tid / CR_SCAN_COLS, j = j0 + jl;      // 8 row parts
+    const bool col_ok = j < vdim;
+    const float * S0 = state + ((int64_t) slot * heads + h) * dim * vdim;
+    for (int idx = tid; idx < dim * CR_SCAN_COLS; idx += 256) {
+        const int i = idx / CR_SCAN_COLS, jj = j0 + idx % CR_SCAN_COLS;
+        Sb[idx] = (jj < vdim && !(word & CM_FRESH)) ? S0[(int64_t) i * vdim + jj] : 0.0f;
+    }
+    int cur = 0;
+    for (int p = 0; p < nsub; p++) {
+        float * blk = scratch + ((int64_t) (sub0 + p) * heads + h) * dim * sw;
+        const bool more = p + 1 < nsub;
+        __syncthreads();                                               // (S of this piece is complete, T of the last one is no longer read)
+        if (more) for (int idx = tid; idx < dim * dim; idx += 256) { const int i = idx / dim, c = idx % dim; Tt[c * tp + i] = blk[(int64_t) i * sw + vdim + c]; }
+        __syncthreads();
+        const float * Sc = Sb + cur * dim * CR_SCAN_COLS;
+        float * Sn = Sb + (cur ^ 1) * dim * CR_SCAN_COLS;
+        for (int i0 = part * 8; i0 < dim; i0 += 64) {
+            float acc[8];
+#pragma unroll
+            for (int r = 0; r < 8; r++) acc[r] = (more && col_ok && i0 + r < dim) ? blk[(int64_t) (i0 + r) * sw + j] : 0.0f;          // L_p, read before S_in(p) takes its place
+            if (col_ok)
+#pragma unroll
+                for (int r = 0; r < 8; r++) if (i0 + r < dim) blk[(int64_t) (i0 + r) * sw + j] = Sc[(i0 + r) * CR_SCAN_COLS + jl];
+            if (!more) continue;
+            for (int c = 0; c < dim; c++) {
+                const float sv = Sc[c * CR_SCAN_COLS + jl];
+                const float * tr = Tt + c * tp + i0;
+#pragma unroll
+                for (int r = 0; r < 8; r++) acc[r] = fmaf(tr[r], sv, acc[r]);      // (rows beyond dim read the pad or the next row of T^T: their sums are dropped)
+            }
+#pragma unroll
+            for (int r = 0; r < 8; r++) if (i0 + r < dim) Sn[(i0 + r) * CR_SCAN_COLS + jl] = acc[r];
+        }
+        cur ^= 1;
+    }
 }
 
 #define CR_LDS_MAX (150 * 1024)
@@ -283,12 +393,19 @@ extern "C" int pi_op_channel_recurrence_reserve(void) {
     static bool done = false;
     if (done) return 0;
     if (cr_reserve_one<8, 0>() || cr_reserve_one<16, 0>() || cr_reserve_one<32, 0>() || cr_reserve_one<8, 1>() || cr_reserve_one<16, 1>() || cr_reserve_one<32, 1>()) return -1;
+    PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_channel_state_scan, hipFuncAttributeMaxDynamicSharedMemorySize, CR_LDS_MAX));
     done = true;
     return 0;
 }
+static int cr_max_pieces(int n_tok, int max_segments) { return n_tok / CR_TB + std::min(n_tok, std::max(1, max_segments)) + 1; }
+// passes of more than 32 tokens cut the runs into pieces that run side by side: floats of scratch they need (0: such a pass is walked in one piece per run)
+extern "C" size_t pi_op_channel_recurrence_scratch_floats(int heads, int dim, int vdim, int n_tok, int max_segments) {
+    return (n_tok <= CR_TB || dim > CR_SCAN_MAXDIM) ? 0 : (size_t) cr_max_pieces(n_tok, max_segments) * heads * dim * (vdim + dim);
+}
 extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_stride, const float * k, int64_t k_stride, const float * v, int64_t v_stride, const float * decay_raw, int64_t decay_stride, int decay_mode,
                                         const float * decay_bias_dev, const float * a_log_dev, const float * beta_raw, int64_t beta_stride, const float * bonus_dev, int qk_unit, float q_mult,
-                                        int heads, int qk_heads, int dim, int vdim, float * state_dev, const int32_t * rec_dev, int n_tok, int max_segments, float * out, int64_t out_stride, void * stream) {
+                                        int heads, int qk_heads, int dim, int vdim, float * state_dev, const int32_t * rec_dev, int n_tok, int max_segments, float * scratch_dev, size_t scratch_floats,
+                                        float * out, int64_t out_stride, void * stream) {
     if (n_tok <= 0) return 0;
     if (rule != PI_RULE_DELTA && rule != PI_RULE_BONUS) { pi_set_error("pi_op_channel_recurrence: rule %d is unknown", rule); return -1; }
     if (qk_heads < 1 || heads % qk_heads) { pi_set_error("pi_op_channel_recurrence: %d heads do not divide over %d query / key heads", heads, qk_heads); return -1; }
@@ -297,21 +414,35 @@ extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_str
     if (max_segments > CR_MAXRUNS) { pi_set_error("pi_op_channel_recurrence: at most %d sequences in a pass", CR_MAXRUNS); return -1; }
     const int dpt = dim <= 8 ? 8 : dim <= 16 ? 16 : 32;                // state values a thread keeps in registers
     int R = 1; while (R * dpt < dim) R *= 2;
-    const int threads = std::min(256, (vdim * R + 63) / 64 * 64);
-    const int cols = threads / R;
-    const dim3 grid((unsigned) heads, (unsigned) ((vdim + cols - 1) / cols), (unsigned) std::max(1, std::min(n_tok, max_segments)));
-    const size_t lds = ((size_t) 3 * CR_TB * dim + (size_t) CR_TB * cols) * sizeof(float);
-    if (lds > CR_LDS_MAX) { pi_set_error("pi_op_channel_recurrence: a key width of %d needs %zu bytes of LDS (at most %d)", dim, lds, CR_LDS_MAX); return -1; }
-    if (lds > 48 * 1024 && pi_op_channel_recurrence_reserve() != 0) return -1;
+    const size_t need = pi_op_channel_recurrence_scratch_floats(heads, dim, vdim, n_tok, max_segments);
+    const bool pieces = need > 0 && scratch_dev && scratch_floats >= need;       // (without scratch a long pass is still right, only serial)
+    const int runs = std::max(1, std::min(n_tok, max_segments));
     const double bytes = 4.0 * n_tok * heads * (3.0 * dim + 2.0 * vdim) + 8.0 * heads * dim * vdim;
     hipStream_t s = (hipStream_t) stream;
     const int nta = std::min(n_tok, PI_KT_MAXNT - 1);
+    auto launch = [&](int mode) -> int {
+        const int ncol = mode == 1 ? vdim + dim : vdim;
+        const int threads = std::min(256, (ncol * R + 63) / 64 * 64);
+        const int cols = threads / R;
+        const dim3 grid((unsigned) heads, (unsigned) ((ncol + cols - 1) / cols), (unsigned) (mode ? cr_max_pieces(n_tok, max_segments) : runs));
+        const size_t lds = ((size_t) 3 * CR_TB * dim + (size_t) CR_TB * cols) * sizeof(float);
+        if (lds > CR_LDS_MAX) { pi_set_error("pi_op_channel_recurrence: a key width of %d needs %zu bytes of LDS (at most %d)", dim, lds, CR_LDS_MAX); return -1; }
+        if (lds > 48 * 1024 && pi_op_channel_recurrence_reserve() != 0) return -1;
 #define CR_GO(D, RL) PI_KT_LAUNCH(PI_KT_ATT, 0, nta, bytes, (k_channel_recurrence<D, RL>), grid, dim3(threads), lds, s, q, q_stride, k, k_stride, v, v_stride, decay_raw, decay_stride, decay_mode, decay_bias_dev, a_log_dev, \
-                                  beta_raw, beta_stride, bonus_dev, qk_unit, q_mult, heads, heads / qk_heads, dim, vdim, R, state_dev, rec_dev, n_tok, out, out_stride, pi_abort_word())
-    if (rule == PI_RULE_DELTA) { if (dpt == 8) CR_GO(8, 0); else if (dpt == 16) CR_GO(16, 0); else CR_GO(32, 0); }
-    else                       { if (dpt == 8) CR_GO(8, 1); else if (dpt == 16) CR_GO(16, 1); else CR_GO(32, 1); }
+                                  beta_raw, beta_stride, bonus_dev, qk_unit, q_mult, heads, heads / qk_heads, dim, vdim, R, state_dev, rec_dev, n_tok, mode, scratch_dev, out, out_stride, pi_abort_word())
+        if (rule == PI_RULE_DELTA) { if (dpt == 8) CR_GO(8, 0); else if (dpt == 16) CR_GO(16, 0); else CR_GO(32, 0); }
+        else                       { if (dpt == 8) CR_GO(8, 1); else if (dpt == 16) CR_GO(16, 1); else CR_GO(32, 1); }
 #undef CR_GO
-    PI_CHECK_LAUNCH(); return 0;
+        PI_CHECK_LAUNCH(); return 0;
+    };
+    if (!pieces) return launch(0);
+    if (launch(1) != 0) return -1;
+    const size_t scan_lds = ((size_t) dim * (dim + 4) + (size_t) 2 * dim * CR_SCAN_COLS) * sizeof(float);
+    if (scan_lds > 48 * 1024 && pi_op_channel_recurrence_reserve() != 0) return -1;
+    PI_KT_LAUNCH(PI_KT_ATT, 0, nta, 4.0 * cr_max_pieces(n_tok, max_segments) * heads * dim * (2.0 * vdim + dim), k_channel_state_scan, dim3((unsigned) heads, (unsigned) ((vdim + CR_SCAN_COLS - 1) / CR_SCAN_COLS), (unsigned) runs),
+                 dim3(256), scan_lds, s, heads, dim, vdim, state_dev, rec_dev, n_tok, scratch_dev, pi_abort_word());
+    PI_CHECK_LAUNCH();
+    return launch(2);
 }
 
 // ---- per-head RMS norm, weight, gate ------------------------------------------------------------------------------------------------------------------------------

@@ -177,7 +177,8 @@ def _declare(lib):
     lib.pi_op_embed_pair.argtypes = [vp, vp, i32, f32, vp, vp, vp, vp]
     lib.pi_op_rms_post.argtypes = [vp, i64, vp, vp, i64, vp, f32, vp, vp, i64, f32, vp, f32, i32, i32, vp, i64, vp, vp, i64, vp]
     lib.pi_op_token_shift.argtypes = [vp, i64, i32, vp, i32, vp, vp, i32, vp, i64, vp]
-    lib.pi_op_channel_recurrence.argtypes = [i32, vp, i64, vp, i64, vp, i64, vp, i64, i32, vp, vp, vp, i64, vp, i32, f32, i32, i32, i32, i32, vp, vp, i32, i32, vp, i64, vp]
+    lib.pi_op_channel_recurrence.argtypes = [i32, vp, i64, vp, i64, vp, i64, vp, i64, i32, vp, vp, vp, i64, vp, i32, f32, i32, i32, i32, i32, vp, vp, i32, i32, vp, sz, vp, i64, vp]
+    lib.pi_op_channel_recurrence_scratch_floats.argtypes = [i32, i32, i32, i32, i32]; lib.pi_op_channel_recurrence_scratch_floats.restype = sz
     lib.pi_op_head_norm_gate.argtypes = [vp, i64, i32, i32, vp, i32, vp, i64, i32, f32, i32, vp, i64, vp]
     lib.pi_op_qkv_prepare_ex.argtypes = [vp, vp, vp, i64, vp, vp, f32, i32, i32, i32, i32, vp, i32, i32, i32, vp, i32, vp, i64, vp, vp, vp, vp, vp]
     lib.pi_op_chunk_attention_ex.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, i64, i32, f32, f32, i32, f32, i32, i32, i32, i32, i32, i32, i32, vp, i64, vp, vp]

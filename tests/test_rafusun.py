@@ -286,8 +286,10 @@ def recurrence_ref(rule, q, k, v, g, beta, bonus, S):
 @pytest.mark.gpu
 @pytest.mark.parametrize("H,G,D,V", [(2, 1, 6, 5), (1, 1, 40, 70), (4, 2, 33, 8), (3, 3, 130, 20), (2, 2, 8, 300), (1, 1, 1, 1)])
 @pytest.mark.parametrize("rule", [DELTA, BONUS])
-def test_channel_recurrence_rules_decays_and_passes(H, G, D, V, rule):
-    """both rules with every way of forming the decays, unit vectors and beta, grouped q / k heads, several sequences per pass, carried and fresh states, passes longer than a tile"""
+@pytest.mark.parametrize("pieces", [False, True])
+def test_channel_recurrence_rules_decays_and_passes(H, G, D, V, rule, pieces):
+    """both rules with every way of forming the decays, unit vectors and beta, grouped q / k heads, several sequences per pass, carried and fresh states, passes longer than a tile —
+    walked token by token (no scratch) and as pieces side by side with a scan of their transition matrices"""
     U, lib = gpu()
     rng = np.random.default_rng(H * 100 + D + V + rule)
     slots = 3
@@ -295,7 +297,7 @@ def test_channel_recurrence_rules_decays_and_passes(H, G, D, V, rule):
     sd = U.Dev((rng.standard_normal((slots, H, D, V)) * 9).astype(np.float32))
     dbias, a_log, bonus = (rng.standard_normal(H * D) - 1).astype(np.float32), (rng.standard_normal(H) * 0.5).astype(np.float32), rng.standard_normal((H, D)).astype(np.float32)
     dbd, ald, bod = U.Dev(dbias), U.Dev(a_log), U.Dev(bonus)
-    plan = [(1, [(1, 4, True)]), (2, [(0, 3, True), (1, 2, False)]), (0, [(2, 37, True), (0, 1, False)]), (2, [(1, 1, False), (0, 35, False), (2, 1, False)])]
+    plan = [(1, [(1, 4, True)]), (2, [(0, 3, True), (1, 2, False)]), (0, [(2, 37, True), (0, 1, False)]), (2, [(1, 1, False), (0, 35, False), (2, 1, False)]), (1, [(2, 64, False), (1, 97, True), (0, 33, False)])]
     for mode, step in plan:
         T = sum(c for _, c, _ in step)
         q, k = rng.standard_normal((T, G * D + 1)).astype(np.float32), rng.standard_normal((T, G * D + 2)).astype(np.float32)
@@ -321,8 +323,11 @@ def test_channel_recurrence_rules_decays_and_passes(H, G, D, V, rule):
                     want[at, h], states[slot][h] = recurrence_ref(rule, qh, kh, v[at, h * V:(h + 1) * V].astype(np.float64), g, O.sigmoid(braw[at, h]), bonus[h].astype(np.float64), states[slot][h])
                 at += 1
         qd, kd, vd, rd, bd, rc, od = U.Dev(q), U.Dev(k), U.Dev(v), U.Dev(raw), U.Dev(braw), U.Dev(np.array(rec, np.int32)), U.Dev(nbytes=4 * T * (H * V + 1))
+        n_scr = int(lib.pi_op_channel_recurrence_scratch_floats(H, D, V, T, slots)) if pieces else 0
+        assert not pieces or T <= 32 or D > 128 or n_scr > 0
+        scr = U.Dev((np.random.default_rng(1).standard_normal(max(n_scr, 4)) * 7).astype(np.float32))          # (garbage: every value the scan and the second walk read was written before)
         L.check(lib.pi_op_channel_recurrence(rule, qd.ptr, G * D + 1, kd.ptr, G * D + 2, vd.ptr, H * V, rd.ptr, H * D + 3, mode, dbd.ptr, ald.ptr, bd.ptr if rule == DELTA else None, H + 1,
-                                             bod.ptr if rule == BONUS else None, int(unit), 0.7 if unit else 1.0, H, G, D, V, sd.ptr, rc.ptr, T, slots, od.ptr, H * V + 1, None))
+                                             bod.ptr if rule == BONUS else None, int(unit), 0.7 if unit else 1.0, H, G, D, V, sd.ptr, rc.ptr, T, slots, scr.ptr if n_scr else None, n_scr, od.ptr, H * V + 1, None))
         got = od.get(np.float32, (T, H * V + 1))[:, :H * V].reshape(T, H, V)
         assert rel_rms(got, want) < 2e-5, (mode, step)
     st = sd.get(np.float32, (slots, H, D, V))
@@ -347,15 +352,17 @@ def test_delta_rule_keeps_a_far_value_and_replaces_it():
     rec = np.zeros(T, np.int32)
     rec[0] |= F
     sd, od = U.Dev(np.full((1, 1, D, V), 7.0, np.float32)), U.Dev(nbytes=4 * T * V)
+    n_scr = int(lib.pi_op_channel_recurrence_scratch_floats(1, D, V, T, 1))                 # (ten pieces side by side: the far row crosses every transition matrix)
+    scr = U.Dev(nbytes=4 * n_scr)
     devs = [U.Dev(a) for a in (q, k, v, raw, braw, rec)]
-    L.check(lib.pi_op_channel_recurrence(DELTA, devs[0].ptr, D, devs[1].ptr, D, devs[2].ptr, V, devs[3].ptr, D, 0, None, None, devs[4].ptr, 1, None, 1, 1.0, 1, 1, D, V, sd.ptr, devs[5].ptr, T, 1, od.ptr, V, None))
+    L.check(lib.pi_op_channel_recurrence(DELTA, devs[0].ptr, D, devs[1].ptr, D, devs[2].ptr, V, devs[3].ptr, D, 0, None, None, devs[4].ptr, 1, None, 1, 1.0, 1, 1, D, V, sd.ptr, devs[5].ptr, T, 1, scr.ptr, n_scr, od.ptr, V, None))
     got = od.get(np.float32, (T, V))
     assert np.allclose(got[0], v[0], atol=1e-5) and np.allclose(got[T - 2], v[T - 2], atol=1e-5)
     assert np.allclose(got[T - 1], v[T - 1], atol=1e-5)                 # the token's own write is what it reads ...
     S = sd.get(np.float32, (D, V))
     assert np.allclose(S[5], v[T - 1], atol=1e-5) and np.allclose(S[1], v[T - 2], atol=1e-5)      # ... and the far row held v[0] until then (S[5] was replaced, not summed)
     devs[4] = U.Dev(np.full((T, 1), -30.0, np.float32))                  # beta = 0: nothing is ever written, the far key reads zero
-    L.check(lib.pi_op_channel_recurrence(DELTA, devs[0].ptr, D, devs[1].ptr, D, devs[2].ptr, V, devs[3].ptr, D, 0, None, None, devs[4].ptr, 1, None, 1, 1.0, 1, 1, D, V, sd.ptr, devs[5].ptr, T, 1, od.ptr, V, None))
+    L.check(lib.pi_op_channel_recurrence(DELTA, devs[0].ptr, D, devs[1].ptr, D, devs[2].ptr, V, devs[3].ptr, D, 0, None, None, devs[4].ptr, 1, None, 1, 1.0, 1, 1, D, V, sd.ptr, devs[5].ptr, T, 1, scr.ptr, n_scr, od.ptr, V, None))
     assert np.abs(od.get(np.float32, (T, V))).max() < 1e-6
 
 
