@@ -278,6 +278,10 @@ PI_API int pi_op_moe_experts_act(const pi_weight * w_up, const pi_weight * w_dow
 /* ---- operators of blocks whose norm comes after the sum, of recurrences with a decay per key channel, and of soft-max attention inside chunks -------------------------------- */
 /* out[t][:] = widen(table[tokens[t]]) * scale + widen(table2[rows2[t]]) (a row outside its table counts as zeros) */
 PI_API int pi_op_embed_pair(const pi_weight * table, const int32_t * tokens_dev, int n_tok, float scale, const pi_weight * table2, const int32_t * rows2_dev, float * out_dev, void * stream);
+/* pi_op_dense over a matrix whose rows fall into n_seg segments that each read an input of their own: rows [g * seg_rows, (g + 1) * seg_rows) read x + g * seg_off, the last segment takes the
+ * remaining rows (projections of DIFFERENT inputs of one width in one launch where the pass has few tokens) */
+PI_API int pi_op_dense_segments(const pi_weight * w, const float * x_dev, int64_t x_stride, int64_t seg_rows, int64_t seg_off, int n_seg, int n_tok, float * out_dev, int64_t out_stride, int act_a, int64_t rows_a,
+                                int act_b, int exact, void * stream);
 /* the end of a sublayer, R(y) = y / sqrt(mean(y^2) + eps):  m = b ? mean_mult * (R(a) * wa + R(b) * wb) : a;  out = R(alpha * x + layer_scale * m) * w  (layer_scale nullable: 1);
  * w_next != NULL: out_next = R(out) * w_next (the norm of whatever reads the stream next).  out may be x.  Rows of at most 8192 values */
 PI_API int pi_op_rms_post(const float * a_dev, int64_t a_stride, const float * wa_dev, const float * b_dev, int64_t b_stride, const float * wb_dev, float mean_mult, const float * layer_scale_dev,

@@ -417,8 +417,8 @@ static bool forward_pre_post_blocks(llama_context * ctx, int n_tok, int n_kv) {
 //   channel delta    ONE projection [q | k | v | a1 | g1 | beta] -> convolution + silu over q | k | v (+ its state) -> the second halves of the low-rank decay and gate projections -> the recurrence
 //                    (unit q / k, sigmoid(beta), the decays formed from their raw values inside the kernel) -> per-head norm * weight * sigmoid(gate) -> output projection
 //   attention + time mix   [q | k | v] -> rotation in neighbouring pairs, then R(.) per head, cache store -> chunked soft-max attention with a sink and capped scores -> W_o;
-//                    token shift (five mixes of the token and the one before it, + its state) -> r, k, v, silu(g), tanh(w1) from their own mixes -> w2 -> the recurrence with a bonus for the token
-//                    itself (decays exp(-exp(. + w0)) formed inside) -> per-head norm * weight * gate -> W_o;   the mixer's result = (R(left) * w_l + R(right) * w_r) / 2, formed by the row kernel
+//                    token shift (five mixes of the token and the one before it, + its state) -> r, k, v, g, tanh(w1) from their own mixes (one matrix in five segments) -> w2 -> the recurrence with a bonus for the token
+//                    itself (decays exp(-exp(. + w0)) formed inside) -> per-head norm * weight * silu(g) -> W_o;   the mixer's result = (R(left) * w_l + R(right) * w_r) / 2, formed by the row kernel
 // Every sublayer ends in ONE row kernel (pi_op_rms_post): [mean of the two normed branches ->] layer scale -> + alpha x -> norm [-> the model's final norm behind the last sublayer].
 static bool forward_post_norm_blocks(llama_context * ctx, int n_tok, int n_kv) {
     llama_model * m = ctx->model;
@@ -453,7 +453,8 @@ static bool forward_post_norm_blocks(llama_context * ctx, int n_tok, int n_kv) {
             const pi_gate_attention & L = H.left; const pi_time_mix & R = H.shift;
             const int64_t pw = L.in_rows(), hd = (int64_t) L.heads * L.dim, hv = (int64_t) L.heads * L.vdim, gd = (int64_t) L.kv_heads * L.dim, inner = R.inner(), mw = (int64_t) 5 * width;
             float * M = P + (size_t) nb * pw;                                                          // the five mixes [r | k | v | g | w] of every token
-            float * Q = A, * O = Q + (size_t) nb * hd, * RK = O + (size_t) nb * hv, * W1 = RK + (size_t) nb * 4 * inner, * WD = W1 + (size_t) nb * R.decay_rank, * O2 = WD + (size_t) nb * inner;
+            const int64_t rkw = 4 * inner + R.decay_rank;                                              // a token's row of [r | k | v | g | tanh(w1)]
+            float * Q = A, * O = Q + (size_t) nb * hd, * RK = O + (size_t) nb * hv, * WD = RK + (size_t) nb * rkw, * O2 = WD + (size_t) nb * inner;
             float * kc = ctx->lat_cache + ctx->lat_off[il], * vc = kc + (size_t) ctx->n_ctx * gd;
             float * S = ctx->rec_state + ctx->rec_off[il], * shift_state = S + (size_t) n_slots * R.matrix_floats();
             // attention branch
@@ -465,16 +466,13 @@ static bool forward_post_norm_blocks(llama_context * ctx, int n_tok, int n_kv) {
             OP_OK(pi_op_dense(W.w_o, O, hv, n_tok, Y, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
             // time-mix branch
             OP_OK(pi_op_token_shift(x, width, width, W.mu, 5, shift_state, ctx->rec_dev, n_tok, M, mw, s));
-            OP_OK(pi_op_dense(W.w_r, M, mw, n_tok, RK, 4 * inner, PI_ACT_NONE, inner, PI_ACT_NONE, ex, s));
-            OP_OK(pi_op_dense(W.w_k, M + width, mw, n_tok, RK + inner, 4 * inner, PI_ACT_NONE, inner, PI_ACT_NONE, ex, s));
-            OP_OK(pi_op_dense(W.w_v, M + 2 * width, mw, n_tok, RK + 2 * inner, 4 * inner, PI_ACT_NONE, inner, PI_ACT_NONE, ex, s));
-            OP_OK(pi_op_dense(W.w_g, M + 3 * width, mw, n_tok, RK + 3 * inner, 4 * inner, PI_ACT_SILU, inner, PI_ACT_SILU, ex, s));
-            OP_OK(pi_op_dense(W.w_w1, M + 4 * width, mw, n_tok, W1, R.decay_rank, PI_ACT_TANH, R.decay_rank, PI_ACT_TANH, ex, s));
-            OP_OK(pi_op_dense(W.w_w2, W1, R.decay_rank, n_tok, WD, inner, PI_ACT_NONE, inner, PI_ACT_NONE, ex, s));
-            OP_OK(pi_op_channel_recurrence(PI_RULE_BONUS, RK, 4 * inner, RK + inner, 4 * inner, RK + 2 * inner, 4 * inner, WD, inner, 1, W.w0, nullptr, nullptr, 0, W.bonus, 0, 1.0f, R.heads, R.heads, R.dim, R.dim,
+            // r | k | v | g | w1 from their own mixes: rows of ONE matrix in five segments; tanh on w1's rows, the gate's silu waits for the head norm
+            OP_OK(pi_op_dense_segments(W.w_r, M, mw, inner, width, 5, n_tok, RK, rkw, PI_ACT_NONE, 4 * inner, PI_ACT_TANH, ex, s));
+            OP_OK(pi_op_dense(W.w_w2, RK + 4 * inner, rkw, n_tok, WD, inner, PI_ACT_NONE, inner, PI_ACT_NONE, ex, s));
+            OP_OK(pi_op_channel_recurrence(PI_RULE_BONUS, RK, rkw, RK + inner, rkw, RK + 2 * inner, rkw, WD, inner, 1, W.w0, nullptr, nullptr, 0, W.bonus, 0, 1.0f, R.heads, R.heads, R.dim, R.dim,
                                            S, ctx->rec_dev, n_tok, n_slots, ctx->rec_scratch, ctx->rec_scratch_floats, O2, inner, s));
             trace(ctx, "rec", (int) il, O2, inner, n_tok);
-            OP_OK(pi_op_head_norm_gate(O2, inner, R.heads, R.dim, W.mix_norm, 1, RK + 3 * inner, 4 * inner, PI_ACT_NONE, eps, n_tok, O2, inner, s));
+            OP_OK(pi_op_head_norm_gate(O2, inner, R.heads, R.dim, W.mix_norm, 1, RK + 3 * inner, rkw, PI_ACT_SILU, eps, n_tok, O2, inner, s));
             OP_OK(pi_op_dense(W.w_o2, O2, inner, n_tok, Y2, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
             yb = Y2;
         } else { ctx->last_error = "blocks with the norm after the sum are built for the channel-delta and the attention + time-mix mixers"; return false; }

@@ -291,8 +291,8 @@ bool llama_model::ensure_loaded_hybrid(int n_positions, std::string & err) {
                 if (!(W.rotary = pi_rotary_table_create(std::max(n_positions, 32), A.rot_dims, A.rot_base))) { err = std::string("rotation table: ") + pi_last_error(); return false; }
                 const int64_t inner = R.inner();
                 if (!(W.mu = L.vectors({ { r + "mu.r", width }, { r + "mu.k", width }, { r + "mu.v", width }, { r + "mu.g", width }, { r + "mu.w", width } }, 0))) return false;
-                if (!(W.w_r = L.matrix({ { r + "r", inner } }, width)) || !(W.w_k = L.matrix({ { r + "k", inner } }, width)) || !(W.w_v = L.matrix({ { r + "v", inner } }, width)) || !(W.w_g = L.matrix({ { r + "g", inner } }, width))) return false;
-                if (!(W.w_w1 = L.matrix({ { r + "w1", R.decay_rank } }, width)) || !(W.w_w2 = L.matrix({ { r + "w2", inner } }, R.decay_rank)) || !(W.w_o2 = L.matrix({ { r + "o", width } }, inner))) return false;
+                if (!(W.w_r = L.matrix({ { r + "r", inner }, { r + "k", inner }, { r + "v", inner }, { r + "g", inner }, { r + "w1", R.decay_rank } }, width))) return false;      // one matrix, five inputs (pi_op_dense_segments)
+                if (!(W.w_w2 = L.matrix({ { r + "w2", inner } }, R.decay_rank)) || !(W.w_o2 = L.matrix({ { r + "o", width } }, inner))) return false;
                 if (!(W.w0 = L.vector(r + "w0", inner)) || !(W.bonus = L.vector2(r + "u", R.heads, R.dim)) || !(W.mix_norm = L.vector(r + "norm", inner)) || !(W.right_out = L.vector(r + "out", width))) return false;
             } else { err = "a block with the norm after the sum has no mixer of kind " + std::to_string((int) H.mixer); return false; }
             if (H.mlp == PI_MLP_DENSE_GEGLU && (!(W.ff_up = L.matrix({ { p + "mlp.gate", H.ff }, { p + "mlp.up", H.ff } }, width)) || !(W.ff_down = L.matrix({ { p + "mlp.down", width } }, H.ff)))) return false;

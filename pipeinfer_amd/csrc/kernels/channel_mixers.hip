@@ -51,8 +51,9 @@ extern "C" int pi_op_embed_pair(const pi_weight * w, const int32_t * tokens, int
 
 // ---- the end of a sublayer whose norm comes after the sum ------------------------------------------------------------------------------------------------
 // per token row:  m = b ? mb * (R(a) * wa + R(b) * wb) : a;   v = alpha * x + ls * m;   out = R(v) * w;   (w_next)  out_next = R(out) * w_next.   R(y) = y / sqrt(mean(y^2) + eps).
-// A thread keeps its NPT values of every row in registers; out may be x.
-template <int NPT>
+// A thread keeps its NPT values of every row in registers; out may be x.  PRE: every input (rows and weight vectors) is loaded before the first block sum, so that the launch makes ONE
+// trip to memory instead of one per stage (rows up to 4096 wide; wider rows would not fit the registers and load stage by stage).
+template <int NPT, bool PRE>
 __global__ void __launch_bounds__(256) k_rms_post(const float * __restrict__ a, int64_t as, const float * __restrict__ wa, const float * __restrict__ b, int64_t bs, const float * __restrict__ wb, float mb,
                                                   const float * __restrict__ ls, const float * __restrict__ x, int64_t xs, float alpha, const float * __restrict__ w, float eps, int n,
                                                   float * __restrict__ out, int64_t os, const float * __restrict__ w_next, float * __restrict__ out_next, int64_t ons, const int32_t * __restrict__ abort_w) {
@@ -60,34 +61,43 @@ __global__ void __launch_bounds__(256) k_rms_post(const float * __restrict__ a, 
     __shared__ float red[4];
     const int t = blockIdx.x, tid = threadIdx.x;
     float m[NPT], v[NPT];
+    float pwa[PRE ? NPT : 1], pwb[PRE ? NPT : 1], pls[PRE ? NPT : 1], px[PRE ? NPT : 1], pw[PRE ? NPT : 1], pwn[PRE ? NPT : 1];
 #pragma unroll
-    for (int j = 0; j < NPT; j++) { const int i = j * 256 + tid; m[j] = i < n ? a[(int64_t) t * as + i] : 0.0f; }
+    for (int j = 0; j < NPT; j++) {
+        const int i = j * 256 + tid;
+        m[j] = i < n ? a[(int64_t) t * as + i] : 0.0f;
+        v[j] = b && i < n ? b[(int64_t) t * bs + i] : 0.0f;
+        if (PRE) {
+            pwa[j] = b && i < n ? wa[i] : 0.0f; pwb[j] = b && i < n ? wb[i] : 0.0f;
+            pls[j] = ls && i < n ? ls[i] : 1.0f; px[j] = i < n ? x[(int64_t) t * xs + i] : 0.0f; pw[j] = i < n ? w[i] : 0.0f; pwn[j] = w_next && i < n ? w_next[i] : 0.0f;
+        }
+    }
     if (b) {
         float sa = 0.0f, sb = 0.0f;
 #pragma unroll
-        for (int j = 0; j < NPT; j++) { const int i = j * 256 + tid; v[j] = i < n ? b[(int64_t) t * bs + i] : 0.0f; sa = fmaf(m[j], m[j], sa); sb = fmaf(v[j], v[j], sb); }
+        for (int j = 0; j < NPT; j++) { sa = fmaf(m[j], m[j], sa); sb = fmaf(v[j], v[j], sb); }
         sa = cm_block_sum(sa, red); sb = cm_block_sum(sb, red);
         const float ia = 1.0f / sqrtf(sa / (float) n + eps), ib = 1.0f / sqrtf(sb / (float) n + eps);
 #pragma unroll
-        for (int j = 0; j < NPT; j++) { const int i = j * 256 + tid; if (i < n) m[j] = mb * (m[j] * ia * wa[i] + v[j] * ib * wb[i]); }
+        for (int j = 0; j < NPT; j++) { const int i = j * 256 + tid; if (i < n) m[j] = mb * (m[j] * ia * (PRE ? pwa[j] : wa[i]) + v[j] * ib * (PRE ? pwb[j] : wb[i])); }
     }
     float ss = 0.0f;
 #pragma unroll
     for (int j = 0; j < NPT; j++) {
         const int i = j * 256 + tid;
-        v[j] = i < n ? fmaf(alpha, x[(int64_t) t * xs + i], (ls ? ls[i] : 1.0f) * m[j]) : 0.0f;
+        v[j] = i < n ? fmaf(alpha, PRE ? px[j] : x[(int64_t) t * xs + i], (PRE ? pls[j] : ls ? ls[i] : 1.0f) * m[j]) : 0.0f;
         ss = fmaf(v[j], v[j], ss);
     }
     ss = cm_block_sum(ss, red);
     const float inv = 1.0f / sqrtf(ss / (float) n + eps);
     float s2 = 0.0f;
 #pragma unroll
-    for (int j = 0; j < NPT; j++) { const int i = j * 256 + tid; if (i < n) { v[j] = v[j] * inv * w[i]; out[(int64_t) t * os + i] = v[j]; s2 = fmaf(v[j], v[j], s2); } }
+    for (int j = 0; j < NPT; j++) { const int i = j * 256 + tid; if (i < n) { v[j] = v[j] * inv * (PRE ? pw[j] : w[i]); out[(int64_t) t * os + i] = v[j]; s2 = fmaf(v[j], v[j], s2); } }
     if (!w_next) return;
     s2 = cm_block_sum(s2, red);
     const float inv2 = 1.0f / sqrtf(s2 / (float) n + eps);
 #pragma unroll
-    for (int j = 0; j < NPT; j++) { const int i = j * 256 + tid; if (i < n) out_next[(int64_t) t * ons + i] = v[j] * inv2 * w_next[i]; }
+    for (int j = 0; j < NPT; j++) { const int i = j * 256 + tid; if (i < n) out_next[(int64_t) t * ons + i] = v[j] * inv2 * (PRE ? pwn[j] : w_next[i]); }
 }
 extern "C" int pi_op_rms_post(const float * a, int64_t a_stride, const float * wa, const float * b, int64_t b_stride, const float * wb, float mean_mult, const float * layer_scale, const float * x, int64_t x_stride,
                               float alpha, const float * w, float eps, int n, int n_tok, float * out, int64_t out_stride, const float * w_next, float * out_next, int64_t out_next_stride, void * stream) {
@@ -96,9 +106,9 @@ extern "C" int pi_op_rms_post(const float * a, int64_t a_stride, const float * w
     if (b && (!wa || !wb)) { pi_set_error("pi_op_rms_post: two inputs need the weights of their norms"); return -1; }
     if (w_next && !out_next) { pi_set_error("pi_op_rms_post: a second norm needs a place for its result"); return -1; }
     const double bytes = 4.0 * n * n_tok * (3.0 + (b ? 1 : 0) + (w_next ? 1 : 0));
-#define RP_GO(N) PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, bytes, k_rms_post<N>, dim3((unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, a, a_stride, wa, b, b_stride, wb, mean_mult, layer_scale, x, x_stride, alpha, w, eps, n, \
+#define RP_GO(N, P) PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, bytes, (k_rms_post<N, P>), dim3((unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, a, a_stride, wa, b, b_stride, wb, mean_mult, layer_scale, x, x_stride, alpha, w, eps, n, \
                               out, out_stride, w_next, out_next, out_next_stride, pi_abort_word())
-    if (n <= 256 * 2) RP_GO(2); else if (n <= 256 * 4) RP_GO(4); else if (n <= 256 * 8) RP_GO(8); else if (n <= 256 * 16) RP_GO(16); else RP_GO(32);
+    if (n <= 256 * 2) RP_GO(2, true); else if (n <= 256 * 4) RP_GO(4, true); else if (n <= 256 * 8) RP_GO(8, true); else if (n <= 256 * 16) RP_GO(16, true); else RP_GO(32, false);
 #undef RP_GO
     PI_CHECK_LAUNCH(); return 0;
 }
@@ -167,9 +177,10 @@ extern "C" int pi_op_token_shift(const float * h, int64_t h_stride, int n, const
 //   bonus:  c = S^T q;  o = c + v (sum_i q_i b_i k_i);  S <- g S + k v
 // A pass of up to CR_TB tokens (or keys too wide for the scan's tile) is ONE launch, mode 0: a piece is a sequence's whole run, S comes from and goes back to HBM.  Longer passes cut
 // every run into pieces of CR_TB tokens that run side by side, because a column's step is affine in the column, s <- A_t s + b_t v_j with A_t the same for every column:
-//   mode 1  every piece but a run's last, with dim extra columns: L_p = the state the piece builds from ZERO, and T_p = A_n .. A_1, whose column c is what the piece makes of the unit
-//           vector e_c with v = 0 — the same walk over a column that starts as e_c — both into scratch [piece][head][dim][vdim + dim]
-//   k_channel_state_scan  per run, piece by piece: S_in(p + 1) = T_p S_in(p) + L_p, S_in(0) = the slot's state (or zero); scratch[p][..][0 .. vdim) <- S_in(p)
+//   mode 1  every piece but a run's last, with extra columns: L_p = the state the piece builds from ZERO, and T_p = A_n .. A_1.  Delta rule: dim extra columns, column c of T_p is what the
+//           piece makes of the unit vector e_c with v = 0 — the same walk over a column that starts as e_c.  Bonus rule: A_t is diagonal, ONE extra column that starts as all ones ends as
+//           the diagonal of T_p.  Both into scratch [piece][head][dim][vdim + extra]
+//   k_channel_state_scan / _diag  per run, piece by piece: S_in(p + 1) = T_p S_in(p) + L_p, S_in(0) = the slot's state (or zero); scratch[p][..][0 .. vdim) <- S_in(p)
 //   mode 2  every piece from its true S_in(p): outputs; a run's last piece leaves the slot's new state
 #define CR_TB 32
 #define CR_MAXRUNS 256
@@ -201,8 +212,9 @@ __global__ void __launch_bounds__(256) k_channel_recurrence(const float * __rest
     __shared__ int seg[4], bnd[CR_MAXRUNS], sorted[CR_MAXRUNS], nbnd;      // seg: first token, length, slot word of this workgroup's piece, whether it is its run's last
     __shared__ float beta_t[CR_TB], dot_t[CR_TB];
     const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
-    const int n_runs = cr_runs(rec, n_tok, bnd, sorted, &nbnd);
-    if (tid == 0) {                               // piece number blockIdx.z of the pass (mode 0: pieces are whole runs)
+    const int n_runs = n_tok == 1 ? 1 : cr_runs(rec, n_tok, bnd, sorted, &nbnd);      // (a single token is its own run: no search, no barrier)
+    if (n_tok == 1) { if (tid == 0) { seg[0] = 0; seg[1] = blockIdx.z == 0 ? 1 : 0; seg[2] = rec[0]; seg[3] = 1; } }
+    else if (tid == 0) {                          // piece number blockIdx.z of the pass (mode 0: pieces are whole runs)
         const int lseg = mode ? CR_TB : 0, want = blockIdx.z;
         int ord = 0;
         seg[1] = 0; seg[2] = -1;
@@ -222,7 +234,8 @@ __global__ void __launch_bounds__(256) k_channel_recurrence(const float * __rest
     if (len == 0 || word < 0 || (mode == 1 && last)) return;
     const int slot = word & ~CM_FRESH;
     const int cols = blockDim.x / R;
-    const int ncol = mode == 1 ? vdim + dim : vdim, sw = vdim + dim;   // columns this launch walks; row stride of a piece's block in scratch
+    const int ext = RULE == 0 ? dim : 1;                              // extra columns of mode 1
+    const int ncol = mode == 1 ? vdim + ext : vdim, sw = vdim + ext;   // columns this launch walks; row stride of a piece's block in scratch
     const int j = blockIdx.y * cols + tid / R, sp = tid % R;
     const bool col_ok = j < ncol;
     const int hq = h / hpg;                                            // the q / k head this head reads
@@ -234,7 +247,7 @@ __global__ void __launch_bounds__(256) k_channel_recurrence(const float * __rest
         const int i = sp * DPT + ii;
         float s0 = 0.0f;
         if (col_ok && i < dim) {
-            if (mode == 1) s0 = j >= vdim && i == j - vdim ? 1.0f : 0.0f;
+            if (mode == 1) s0 = j >= vdim && (RULE == 1 || i == j - vdim) ? 1.0f : 0.0f;
             else if (mode == 2) s0 = S_scr[(int64_t) i * sw + j];
             else if (!(word & CM_FRESH)) s0 = S_hbm[(int64_t) i * vdim + j];
         }
@@ -327,7 +340,7 @@ __global__ void __launch_bounds__(256) k_channel_recurrence(const float * __rest
 
 // grid (head, blocks of CR_SCAN_COLS value columns, run): per piece p of the run, in order: scratch[p] holds [L_p | T_p] coming in and S_in(p) (in L_p's place) going out.
 // A workgroup keeps its columns of S in LDS (two buffers) and T_p transposed ([c][i], so that a thread's rows are neighbours); thread (column j, row part): 8 rows at a time in registers.
-#define CR_SCAN_COLS 32
+template <int CR_SCAN_COLS>
 __global__ void __launch_bounds__(256) k_channel_state_scan(int heads, int dim, int vdim, const float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, float * __restrict__ scratch,
                                                             const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
@@ -350,7 +363,7 @@ __global__ void __launch_bounds__(256) k_channel_state_scan(int heads, int dim, 
     if (nsub == 0 || word < 0) return;
     const int slot = word & ~CM_FRESH, sw = vdim + dim, tp = dim + 4;
     float * Tt = lds, * Sb = Tt + dim * tp;
-    const int jl = tid % CR_SCAN_COLS, part = tid / CR_SCAN_COLS, j = j0 + jl;      // 8 row parts
+    const int jl = tid % CR_SCAN_COLS, part = tid / CR_SCAN_COLS, j = j0 + jl, pstep = 8 * (256 / CR_SCAN_COLS);      // row parts of 8 rows
     const bool col_ok = j < vdim;
     const float * S0 = state + ((int64_t) slot * heads + h) * dim * vdim;
     for (int idx = tid; idx < dim * CR_SCAN_COLS; idx += 256) {
@@ -366,7 +379,7 @@ __global__ void __launch_bounds__(256) k_channel_state_scan(int heads, int dim, 
         __syncthreads();
         const float * Sc = Sb + cur * dim * CR_SCAN_COLS;
         float * Sn = Sb + (cur ^ 1) * dim * CR_SCAN_COLS;
-        for (int i0 = part * 8; i0 < dim; i0 += 64) {
+        for (int i0 = part * 8; i0 < dim; i0 += pstep) {
             float acc[8];
 #pragma unroll
             for (int r = 0; r < 8; r++) acc[r] = (more && col_ok && i0 + r < dim) ? blk[(int64_t) (i0 + r) * sw + j] : 0.0f;          // L_p, read before S_in(p) takes its place
@@ -387,19 +400,62 @@ __global__ void __launch_bounds__(256) k_channel_state_scan(int heads, int dim, 
     }
 }
 
+// the same chain where T_p is diagonal (bonus rule): scratch[p] holds [L_p | diag T_p] ([dim][vdim + 1]).  grid (head, blocks over dim * vdim, run): eight pieces' loads in flight, the chain in registers
+__global__ void __launch_bounds__(256) k_channel_state_scan_diag(int heads, int dim, int vdim, const float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, float * __restrict__ scratch,
+                                                                 const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    __shared__ int seg[3], bnd[CR_MAXRUNS], sorted[CR_MAXRUNS], nbnd;
+    const int tid = threadIdx.x, h = blockIdx.x;
+    const int n_runs = cr_runs(rec, n_tok, bnd, sorted, &nbnd);
+    if (tid == 0) {
+        int ord = 0;
+        seg[0] = -1; seg[2] = 0;
+        for (int r = 0; r < n_runs; r++) {
+            const int t = sorted[r], e = r + 1 < n_runs ? sorted[r + 1] : n_tok;
+            const int ns = (e - t + CR_TB - 1) / CR_TB;
+            if (r == (int) blockIdx.z) { seg[0] = rec[t]; seg[1] = ord; seg[2] = ns; break; }
+            ord += ns;
+        }
+    }
+    __syncthreads();
+    const int word = seg[0], sub0 = seg[1], nsub = seg[2];
+    if (nsub == 0 || word < 0) return;
+    const int64_t per = (int64_t) dim * vdim, idx = (int64_t) blockIdx.y * 256 + tid;
+    if (idx >= per) return;
+    const int i = (int) (idx / vdim), j = (int) (idx % vdim), sw = vdim + 1;
+    float run = (word & CM_FRESH) ? 0.0f : state[((int64_t) (word & ~CM_FRESH) * heads + h) * per + idx];
+    for (int p0 = 0; p0 < nsub; p0 += 8) {
+        float lp[8], tp[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const float * blk = scratch + ((int64_t) (sub0 + p0 + u) * heads + h) * dim * sw + (int64_t) i * sw;
+            const bool more = p0 + u < nsub - 1;
+            lp[u] = more ? blk[j] : 0.0f; tp[u] = more ? blk[vdim] : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+            if (p0 + u < nsub) {
+                scratch[((int64_t) (sub0 + p0 + u) * heads + h) * dim * sw + (int64_t) i * sw + j] = run;
+                run = fmaf(tp[u], run, lp[u]);
+            }
+    }
+}
+
 #define CR_LDS_MAX (150 * 1024)
 template <int DPT, int RULE> static int cr_reserve_one() { PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_channel_recurrence<DPT, RULE>, hipFuncAttributeMaxDynamicSharedMemorySize, CR_LDS_MAX)); return 0; }
 extern "C" int pi_op_channel_recurrence_reserve(void) {
     static bool done = false;
     if (done) return 0;
     if (cr_reserve_one<8, 0>() || cr_reserve_one<16, 0>() || cr_reserve_one<32, 0>() || cr_reserve_one<8, 1>() || cr_reserve_one<16, 1>() || cr_reserve_one<32, 1>()) return -1;
-    PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_channel_state_scan, hipFuncAttributeMaxDynamicSharedMemorySize, CR_LDS_MAX));
+    PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_channel_state_scan<8>, hipFuncAttributeMaxDynamicSharedMemorySize, CR_LDS_MAX));
+    PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_channel_state_scan<16>, hipFuncAttributeMaxDynamicSharedMemorySize, CR_LDS_MAX));
+    PI_CHECK_HIP(hipFuncSetAttribute((const void *) k_channel_state_scan<32>, hipFuncAttributeMaxDynamicSharedMemorySize, CR_LDS_MAX));
     done = true;
     return 0;
 }
 static int cr_max_pieces(int n_tok, int max_segments) { return n_tok / CR_TB + std::min(n_tok, std::max(1, max_segments)) + 1; }
 // passes of more than 32 tokens cut the runs into pieces that run side by side: floats of scratch they need (0: such a pass is walked in one piece per run)
-extern "C" size_t pi_op_channel_recurrence_scratch_floats(int heads, int dim, int vdim, int n_tok, int max_segments) {
+extern "C" size_t pi_op_channel_recurrence_scratch_floats(int heads, int dim, int vdim, int n_tok, int max_segments) {      // (sized for the delta rule, which needs more)
     return (n_tok <= CR_TB || dim > CR_SCAN_MAXDIM) ? 0 : (size_t) cr_max_pieces(n_tok, max_segments) * heads * dim * (vdim + dim);
 }
 extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_stride, const float * k, int64_t k_stride, const float * v, int64_t v_stride, const float * decay_raw, int64_t decay_stride, int decay_mode,
@@ -421,7 +477,7 @@ extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_str
     hipStream_t s = (hipStream_t) stream;
     const int nta = std::min(n_tok, PI_KT_MAXNT - 1);
     auto launch = [&](int mode) -> int {
-        const int ncol = mode == 1 ? vdim + dim : vdim;
+        const int ncol = mode == 1 ? vdim + (rule == PI_RULE_DELTA ? dim : 1) : vdim;
         const int threads = std::min(256, (ncol * R + 63) / 64 * 64);
         const int cols = threads / R;
         const dim3 grid((unsigned) heads, (unsigned) ((ncol + cols - 1) / cols), (unsigned) (mode ? cr_max_pieces(n_tok, max_segments) : runs));
@@ -437,10 +493,22 @@ extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_str
     };
     if (!pieces) return launch(0);
     if (launch(1) != 0) return -1;
-    const size_t scan_lds = ((size_t) dim * (dim + 4) + (size_t) 2 * dim * CR_SCAN_COLS) * sizeof(float);
-    if (scan_lds > 48 * 1024 && pi_op_channel_recurrence_reserve() != 0) return -1;
-    PI_KT_LAUNCH(PI_KT_ATT, 0, nta, 4.0 * cr_max_pieces(n_tok, max_segments) * heads * dim * (2.0 * vdim + dim), k_channel_state_scan, dim3((unsigned) heads, (unsigned) ((vdim + CR_SCAN_COLS - 1) / CR_SCAN_COLS), (unsigned) runs),
-                 dim3(256), scan_lds, s, heads, dim, vdim, state_dev, rec_dev, n_tok, scratch_dev, pi_abort_word());
+    const int n_pieces = cr_max_pieces(n_tok, max_segments);
+    if (rule == PI_RULE_BONUS) {
+        PI_KT_LAUNCH(PI_KT_ATT, 0, nta, 12.0 * n_pieces * heads * dim * vdim, k_channel_state_scan_diag, dim3((unsigned) heads, (unsigned) (((int64_t) dim * vdim + 255) / 256), (unsigned) runs), dim3(256), 0, s,
+                     heads, dim, vdim, state_dev, rec_dev, n_tok, scratch_dev, pi_abort_word());
+    } else {
+        // columns per workgroup: as few as it takes to put a workgroup on every compute unit (each one re-reads the transition matrices, which the others' reads keep in L2)
+        int sc = 32;
+        while (sc > 8 && (int64_t) heads * ((vdim + sc - 1) / sc) * runs < 256) sc >>= 1;
+        const size_t scan_lds = ((size_t) dim * (dim + 4) + (size_t) 2 * dim * sc) * sizeof(float);
+        if (scan_lds > 48 * 1024 && pi_op_channel_recurrence_reserve() != 0) return -1;
+        const dim3 sgrid((unsigned) heads, (unsigned) ((vdim + sc - 1) / sc), (unsigned) runs);
+        const double sbytes = 4.0 * n_pieces * heads * dim * (2.0 * vdim + dim);
+#define CR_SCAN(C) PI_KT_LAUNCH(PI_KT_ATT, 0, nta, sbytes, k_channel_state_scan<C>, sgrid, dim3(256), scan_lds, s, heads, dim, vdim, state_dev, rec_dev, n_tok, scratch_dev, pi_abort_word())
+        if (sc == 8) CR_SCAN(8); else if (sc == 16) CR_SCAN(16); else CR_SCAN(32);
+#undef CR_SCAN
+    }
     PI_CHECK_LAUNCH();
     return launch(2);
 }

@@ -47,11 +47,12 @@ __global__ void k_embed(const uint16_t * __restrict__ table, int64_t width, int6
 // VW weights per lane and step (8: one 16-byte load, 4: 8 bytes, 1: any K and alignment)
 template <int TT, int VW, bool EXACT>
 __global__ void __launch_bounds__(256) k_dense_rows(const uint16_t * __restrict__ W, int64_t K, int64_t N, const float * __restrict__ X, int64_t xs, int T, float * __restrict__ Y, int64_t ys,
-                                                    int act_a, int64_t rows_a, int act_b, const int32_t * __restrict__ abort_w) {
+                                                    int act_a, int64_t rows_a, int act_b, int64_t seg_rows, int64_t seg_off, int seg_last, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 0)) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t row = (int64_t) blockIdx.x * 4 + wave;
     if (row >= N) return;
+    if (seg_rows > 0) X += min(row / seg_rows, (int64_t) seg_last) * seg_off;       // rows in segments of seg_rows (the last one takes the rest), every segment with an input of its own
     const int t0 = blockIdx.y * TT;
     float acc[TT];
 #pragma unroll
@@ -213,13 +214,13 @@ extern "C" int pi_op_embed(const pi_weight * w, const int32_t * tokens, int n_to
 static int dense_mfma_min_tokens() { static const int v = getenv("PI_DENSE_MFMA_MIN") ? atoi(getenv("PI_DENSE_MFMA_MIN")) : 16; return v; }
 
 template <int VW, bool EXACT>
-static void launch_rows(const pi_weight * w, const float * x, int64_t xs, int n_tok, float * out, int64_t os, int act_a, int64_t rows_a, int act_b, hipStream_t s, double bytes) {
+static void launch_rows(const pi_weight * w, const float * x, int64_t xs, int n_tok, float * out, int64_t os, int act_a, int64_t rows_a, int act_b, hipStream_t s, double bytes, int64_t seg_rows = 0, int64_t seg_off = 0, int seg_last = 0) {
     const uint16_t * W = (const uint16_t *) w->p0;
     const unsigned gx = (unsigned) ((w->ne1 + 3) / 4);
     const int nt_acct = std::min(n_tok, PI_KT_MAXNT - 1);
-    if (n_tok == 1)      PI_KT_LAUNCH(PI_KT_MATVEC, PI_BF16, nt_acct, bytes, (k_dense_rows<1, VW, EXACT>), dim3(gx, 1), dim3(256), 0, s, W, w->ne0, w->ne1, x, xs, n_tok, out, os, act_a, rows_a, act_b, pi_abort_word());
-    else if (n_tok <= 4) PI_KT_LAUNCH(PI_KT_MATVEC, PI_BF16, nt_acct, bytes, (k_dense_rows<4, VW, EXACT>), dim3(gx, 1), dim3(256), 0, s, W, w->ne0, w->ne1, x, xs, n_tok, out, os, act_a, rows_a, act_b, pi_abort_word());
-    else PI_KT_LAUNCH(PI_KT_MATVEC, PI_BF16, nt_acct, bytes, (k_dense_rows<8, VW, EXACT>), dim3(gx, (unsigned) ((n_tok + 7) / 8)), dim3(256), 0, s, W, w->ne0, w->ne1, x, xs, n_tok, out, os, act_a, rows_a, act_b, pi_abort_word());
+    if (n_tok == 1)      PI_KT_LAUNCH(PI_KT_MATVEC, PI_BF16, nt_acct, bytes, (k_dense_rows<1, VW, EXACT>), dim3(gx, 1), dim3(256), 0, s, W, w->ne0, w->ne1, x, xs, n_tok, out, os, act_a, rows_a, act_b, seg_rows, seg_off, seg_last, pi_abort_word());
+    else if (n_tok <= 4) PI_KT_LAUNCH(PI_KT_MATVEC, PI_BF16, nt_acct, bytes, (k_dense_rows<4, VW, EXACT>), dim3(gx, 1), dim3(256), 0, s, W, w->ne0, w->ne1, x, xs, n_tok, out, os, act_a, rows_a, act_b, seg_rows, seg_off, seg_last, pi_abort_word());
+    else PI_KT_LAUNCH(PI_KT_MATVEC, PI_BF16, nt_acct, bytes, (k_dense_rows<8, VW, EXACT>), dim3(gx, (unsigned) ((n_tok + 7) / 8)), dim3(256), 0, s, W, w->ne0, w->ne1, x, xs, n_tok, out, os, act_a, rows_a, act_b, seg_rows, seg_off, seg_last, pi_abort_word());
 }
 
 extern "C" int pi_op_dense(const pi_weight * w, const float * x, int64_t x_stride, int n_tok, float * out, int64_t out_stride, int act_a, int64_t rows_a, int act_b, int exact, void * stream) {
@@ -246,4 +247,33 @@ extern "C" int pi_op_dense(const pi_weight * w, const float * x, int64_t x_strid
     else if (al8)         { if (exact) launch_rows<4, true>(w, x, x_stride, n_tok, out, out_stride, act_a, rows_a, act_b, s, bytes); else launch_rows<4, false>(w, x, x_stride, n_tok, out, out_stride, act_a, rows_a, act_b, s, bytes); }
     else                  { if (exact) launch_rows<1, true>(w, x, x_stride, n_tok, out, out_stride, act_a, rows_a, act_b, s, bytes); else launch_rows<1, false>(w, x, x_stride, n_tok, out, out_stride, act_a, rows_a, act_b, s, bytes); }
     PI_CHECK_LAUNCH(); return 0;
+}
+
+// one matrix whose rows fall into segments that each read an input of their own: rows [g * seg_rows, (g + 1) * seg_rows) read x + g * seg_off (g < n_seg - 1; the last segment takes the remaining
+// rows).  Few tokens (the mat-vec kernel): ONE launch; wider passes take a matrix-core launch per segment
+extern "C" int pi_op_dense_segments(const pi_weight * w, const float * x, int64_t x_stride, int64_t seg_rows, int64_t seg_off, int n_seg, int n_tok, float * out, int64_t out_stride, int act_a, int64_t rows_a,
+                                    int act_b, int exact, void * stream) {
+    if (!w || w->type != PI_BF16) { pi_set_error("pi_op_dense: the weight must be bfloat16"); return -1; }
+    if (n_tok <= 0 || w->ne1 <= 0) return 0;
+    if (n_seg < 1 || seg_rows < 1 || (int64_t) (n_seg - 1) * seg_rows >= w->ne1) { pi_set_error("pi_op_dense_segments: %d segments of %lld rows do not fit %lld rows", n_seg, (long long) seg_rows, (long long) w->ne1); return -1; }
+    const int64_t K = w->ne0;
+    if (x_stride < (int64_t) (n_seg - 1) * seg_off + K || out_stride < w->ne1) { pi_set_error("pi_op_dense_segments: row strides below the sizes"); return -1; }
+    const bool al16 = K % 8 == 0 && ((uintptr_t) w->p0 % 16) == 0 && ((uintptr_t) x % 16) == 0 && x_stride % 4 == 0 && seg_off % 4 == 0;
+    if (exact || !al16 || n_tok < dense_mfma_min_tokens()) {
+        const bool al8 = K % 4 == 0 && ((uintptr_t) w->p0 % 8) == 0 && ((uintptr_t) x % 16) == 0 && x_stride % 4 == 0 && seg_off % 4 == 0;
+        const double bytes = 2.0 * K * w->ne1 + 4.0 * n_tok * (n_seg * K + w->ne1);
+        hipStream_t s = (hipStream_t) stream;
+        if (al16 && K >= 512) { if (exact) launch_rows<8, true>(w, x, x_stride, n_tok, out, out_stride, act_a, rows_a, act_b, s, bytes, seg_rows, seg_off, n_seg - 1); else launch_rows<8, false>(w, x, x_stride, n_tok, out, out_stride, act_a, rows_a, act_b, s, bytes, seg_rows, seg_off, n_seg - 1); }
+        else if (al8)         { if (exact) launch_rows<4, true>(w, x, x_stride, n_tok, out, out_stride, act_a, rows_a, act_b, s, bytes, seg_rows, seg_off, n_seg - 1); else launch_rows<4, false>(w, x, x_stride, n_tok, out, out_stride, act_a, rows_a, act_b, s, bytes, seg_rows, seg_off, n_seg - 1); }
+        else                  { if (exact) launch_rows<1, true>(w, x, x_stride, n_tok, out, out_stride, act_a, rows_a, act_b, s, bytes, seg_rows, seg_off, n_seg - 1); else launch_rows<1, false>(w, x, x_stride, n_tok, out, out_stride, act_a, rows_a, act_b, s, bytes, seg_rows, seg_off, n_seg - 1); }
+        PI_CHECK_LAUNCH(); return 0;
+    }
+    for (int g = 0; g < n_seg; g++) {                                  // a view of the segment's rows
+        pi_weight view = *w;
+        const int64_t r0 = (int64_t) g * seg_rows;
+        view.p0 = w->p0 + (size_t) r0 * K * 2; view.ne1 = g == n_seg - 1 ? w->ne1 - r0 : seg_rows;
+        const int64_t ra = std::max<int64_t>(0, std::min<int64_t>(view.ne1, rows_a - r0));
+        if (pi_op_dense(&view, x + g * seg_off, x_stride, n_tok, out + r0, out_stride, act_a, ra, act_b, exact, stream) != 0) return -1;
+    }
+    return 0;
 }

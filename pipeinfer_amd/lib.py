@@ -174,6 +174,7 @@ def _declare(lib):
     lib.pi_op_moe_experts_act.argtypes = [vp, vp, i32, i32, i32, vp, i64, vp, vp, i32, i32, i32, vp, vp, i64, vp]
     lib.pi_op_moe_experts_grouped_act.argtypes = [vp, vp, i32, i32, i32, vp, i64, vp, vp, i32, i32, vp, vp, vp, vp, i64, vp]
     # blocks with the norm after the sum, recurrences with a decay per key channel, soft-max attention in chunks
+    lib.pi_op_dense_segments.argtypes = [vp, vp, i64, i64, i64, i32, i32, vp, i64, i32, i64, i32, i32, vp]
     lib.pi_op_embed_pair.argtypes = [vp, vp, i32, f32, vp, vp, vp, vp]
     lib.pi_op_rms_post.argtypes = [vp, i64, vp, vp, i64, vp, f32, vp, vp, i64, f32, vp, f32, i32, i32, vp, i64, vp, vp, i64, vp]
     lib.pi_op_token_shift.argtypes = [vp, i64, i32, vp, i32, vp, vp, i32, vp, i64, vp]

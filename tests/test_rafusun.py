@@ -215,7 +215,29 @@ def test_dense_epilogues_tanh_and_gelu():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("n", [5, 96, 300, 1000, 2100])
+@pytest.mark.parametrize("T", [1, 5, 40])
+@pytest.mark.parametrize("exact", [1, 0])
+def test_dense_rows_in_segments_with_inputs_of_their_own(T, exact):
+    """one matrix, five inputs: rows of a segment read their own input (the mat-vec kernel in one launch, wider passes segment by segment on the matrix cores); the last segment is shorter"""
+    U, lib = gpu()
+    rng = np.random.default_rng(T)
+    K, seg, last, n_seg = 64, 24, 8, 5
+    rows = (n_seg - 1) * seg + last
+    W = O.bf16_round(rng.standard_normal((rows, K)).astype(np.float32))
+    x = O.bf16_round(rng.standard_normal((T, n_seg * K + 4)).astype(np.float32))            # (bfloat16 values: both precisions give the same products)
+    w, xd, od = upload_bf16(lib, W), U.Dev(x), U.Dev(nbytes=4 * T * (rows + 1))
+    L.check(lib.pi_op_dense_segments(w, xd.ptr, n_seg * K + 4, seg, K, n_seg, T, od.ptr, rows + 1, NONE, (n_seg - 1) * seg, TANH, exact, None))
+    want = np.zeros((T, rows))
+    for g in range(n_seg):
+        r0, r1 = g * seg, min((g + 1) * seg, rows)
+        z = x[:, g * K:(g + 1) * K].astype(np.float64) @ W[r0:r1].T.astype(np.float64)
+        want[:, r0:r1] = np.tanh(z) if g == n_seg - 1 else z
+    assert rel_rms(od.get(np.float32, (T, rows + 1))[:, :rows], want) < 2e-6
+    lib.pi_weight_free(w)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n", [5, 96, 300, 1000, 2100, 4100])
 def test_sublayer_end_with_one_and_two_inputs(n):
     """layer scale, + alpha x, norm; the mean of two normed branches in front; the second norm behind; in place"""
     U, lib = gpu()
