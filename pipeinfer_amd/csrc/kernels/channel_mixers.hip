@@ -176,13 +176,14 @@ extern "C" int pi_op_token_shift(const float * h, int64_t h_stride, int n, const
 //   delta:  S <- g S;  a = S^T k, c = S^T q (one pass over the registers);  u = beta (v - a);  o = c + u (k . q);  S <- S + k u
 //   bonus:  c = S^T q;  o = c + v (sum_i q_i b_i k_i);  S <- g S + k v
 // A pass of up to CR_TB tokens (or keys too wide for the scan's tile) is ONE launch, mode 0: a piece is a sequence's whole run, S comes from and goes back to HBM.  Longer passes cut
-// every run into pieces of CR_TB tokens that run side by side, because a column's step is affine in the column, s <- A_t s + b_t v_j with A_t the same for every column:
+// every run into pieces of CR_PIECE tokens that run side by side, because a column's step is affine in the column, s <- A_t s + b_t v_j with A_t the same for every column:
 //   mode 1  every piece but a run's last, with extra columns: L_p = the state the piece builds from ZERO, and T_p = A_n .. A_1.  Delta rule: dim extra columns, column c of T_p is what the
 //           piece makes of the unit vector e_c with v = 0 — the same walk over a column that starts as e_c.  Bonus rule: A_t is diagonal, ONE extra column that starts as all ones ends as
 //           the diagonal of T_p.  Both into scratch [piece][head][dim][vdim + extra]
 //   k_channel_state_scan / _diag  per run, piece by piece: S_in(p + 1) = T_p S_in(p) + L_p, S_in(0) = the slot's state (or zero); scratch[p][..][0 .. vdim) <- S_in(p)
 //   mode 2  every piece from its true S_in(p): outputs; a run's last piece leaves the slot's new state
-#define CR_TB 32
+#define CR_TB 32                                  // tokens staged in LDS at a time
+#define CR_PIECE 64                               // tokens of a piece of a long pass (two tiles: half the pieces for the scan to chain, the same LDS)
 #define CR_MAXRUNS 256
 #define CR_SCAN_MAXDIM 128                        // widest key whose transition matrix the scan keeps in LDS
 // the pass's runs in order (a run: the consecutive tokens of one slot): every thread looks at its own tokens for a run's first one, the few found are ranked by position.  first[r] in `sorted`
@@ -201,21 +202,23 @@ static __device__ __forceinline__ int cr_runs(const int32_t * __restrict__ rec, 
     __syncthreads();
     return n;
 }
+// (amdgpu_waves_per_eu(1, 2): the kernel is a chain of dependent steps per token, what helps is having a token's LDS reads in flight together, which takes registers; the compiler's default
+// aims at eight waves per SIMD, keeps under 64 registers and then waits for every read on its own: 3.4 us per token, measured)
 template <int DPT, int RULE>
-__global__ void __launch_bounds__(256) k_channel_recurrence(const float * __restrict__ q, int64_t qs, const float * __restrict__ k, int64_t ks, const float * __restrict__ v, int64_t vs,
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) k_channel_recurrence(const float * __restrict__ q, int64_t qs, const float * __restrict__ k, int64_t ks, const float * __restrict__ v, int64_t vs,
                                                             const float * __restrict__ draw, int64_t ds, int decay_mode, const float * __restrict__ dbias, const float * __restrict__ a_log,
                                                             const float * __restrict__ braw, int64_t bs, const float * __restrict__ bonus, int qk_unit, float q_mult,
                                                             int heads, int hpg, int dim, int vdim, int R, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, int mode,
                                                             float * __restrict__ scratch, float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
-    extern __shared__ float lds[];                // q [CR_TB][dim] | k [CR_TB][dim] | g [CR_TB][dim] | v [CR_TB][cols]
+    extern __shared__ float lds[];                // q [CR_TB][dp] | k [CR_TB][dp] | g [CR_TB][dp] | v [CR_TB][cols];  a row is R parts of DPT values, DPT + 4 floats apart (the parts of one wave-wide read then fall into different banks), dp = R * (DPT + 4); rows end in zeros so that the token loop needs no bounds
     __shared__ int seg[4], bnd[CR_MAXRUNS], sorted[CR_MAXRUNS], nbnd;      // seg: first token, length, slot word of this workgroup's piece, whether it is its run's last
     __shared__ float beta_t[CR_TB], dot_t[CR_TB];
     const int h = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nw = blockDim.x >> 6;
     const int n_runs = n_tok == 1 ? 1 : cr_runs(rec, n_tok, bnd, sorted, &nbnd);      // (a single token is its own run: no search, no barrier)
     if (n_tok == 1) { if (tid == 0) { seg[0] = 0; seg[1] = blockIdx.z == 0 ? 1 : 0; seg[2] = rec[0]; seg[3] = 1; } }
     else if (tid == 0) {                          // piece number blockIdx.z of the pass (mode 0: pieces are whole runs)
-        const int lseg = mode ? CR_TB : 0, want = blockIdx.z;
+        const int lseg = mode ? CR_PIECE : 0, want = blockIdx.z;
         int ord = 0;
         seg[1] = 0; seg[2] = -1;
         for (int r = 0; r < n_runs; r++) {
@@ -253,21 +256,25 @@ __global__ void __launch_bounds__(256) k_channel_recurrence(const float * __rest
         }
         S[ii] = s0;
     }
-    float * qt = lds, * kt = qt + CR_TB * dim, * gt = kt + CR_TB * dim, * vt = gt + CR_TB * dim;
+    const int dp = R * (DPT + 4);
+    float * qt = lds, * kt = qt + CR_TB * dp, * gt = kt + CR_TB * dp, * vt = gt + CR_TB * dp;
     const float ah = decay_mode == 2 ? expf(a_log[h]) : 0.0f;
-    const bool dim4 = (dim & 3) == 0;
     for (int t0 = 0; t0 < len; t0 += CR_TB) {
         const int nt = min(CR_TB, len - t0);
         __syncthreads();
-        for (int idx = tid; idx < nt * dim; idx += blockDim.x) {
-            const int tt = idx / dim, i = idx % dim;
+        for (int idx = tid; idx < nt * R * DPT; idx += blockDim.x) {
+            const int tt = idx / (R * DPT), i = idx % (R * DPT);
             const int64_t tok = first + t0 + tt;
-            qt[idx] = q[tok * qs + (int64_t) hq * dim + i];
-            kt[idx] = k[tok * ks + (int64_t) hq * dim + i];
-            float d = draw[tok * ds + (int64_t) h * dim + i];
-            if (decay_mode == 1) d = expf(-expf(d + (dbias ? dbias[h * dim + i] : 0.0f)));
-            else if (decay_mode == 2) d = expf(-ah * cm_softplus(d + (dbias ? dbias[h * dim + i] : 0.0f)));
-            gt[idx] = d;
+            float qv = 0.0f, kv = 0.0f, d = 0.0f;
+            if (i < dim) {
+                qv = q[tok * qs + (int64_t) hq * dim + i];
+                kv = k[tok * ks + (int64_t) hq * dim + i];
+                d = draw[tok * ds + (int64_t) h * dim + i];
+                if (decay_mode == 1) d = expf(-expf(d + (dbias ? dbias[h * dim + i] : 0.0f)));
+                else if (decay_mode == 2) d = expf(-ah * cm_softplus(d + (dbias ? dbias[h * dim + i] : 0.0f)));
+            }
+            const int at = tt * dp + i / DPT * (DPT + 4) + i % DPT;
+            qt[at] = qv; kt[at] = kv; gt[at] = d;
         }
         if (tid < nt) beta_t[tid] = braw ? cm_sigmoid(braw[(int64_t) (first + t0 + tid) * bs + h]) : 1.0f;
         for (int idx = tid; idx < nt * cols; idx += blockDim.x) {
@@ -276,55 +283,47 @@ __global__ void __launch_bounds__(256) k_channel_recurrence(const float * __rest
         }
         __syncthreads();
         for (int tt = wave; tt < nt; tt += nw) {                          // a wave per token: unit vectors, then the token's scalar (k . q, or sum q b k)
-            float * qr = qt + tt * dim, * kr = kt + tt * dim;
+            float * qr = qt + tt * dp, * kr = kt + tt * dp;
+            auto at = [&](int i) { return i / DPT * (DPT + 4) + i % DPT; };
             if (qk_unit) {
                 float sq = 0.0f, sk = 0.0f;
-                for (int i = lane; i < dim; i += 64) { sq = fmaf(qr[i], qr[i], sq); sk = fmaf(kr[i], kr[i], sk); }
+                for (int i = lane; i < dim; i += 64) { sq = fmaf(qr[at(i)], qr[at(i)], sq); sk = fmaf(kr[at(i)], kr[at(i)], sk); }
                 const float iq = q_mult / sqrtf(pi_lanes_sum<64>(sq) + 1e-6f), ik = 1.0f / sqrtf(pi_lanes_sum<64>(sk) + 1e-6f);
-                for (int i = lane; i < dim; i += 64) { qr[i] *= iq; kr[i] *= ik; }
-            } else if (q_mult != 1.0f) for (int i = lane; i < dim; i += 64) qr[i] *= q_mult;
+                for (int i = lane; i < dim; i += 64) { qr[at(i)] *= iq; kr[at(i)] *= ik; }
+            } else if (q_mult != 1.0f) for (int i = lane; i < dim; i += 64) qr[at(i)] *= q_mult;
             float d = 0.0f;
-            for (int i = lane; i < dim; i += 64) d = fmaf(RULE == 1 && bonus ? qr[i] * bonus[h * dim + i] : qr[i], kr[i], d);      // (a lane re-reads only what it wrote itself)
+            for (int i = lane; i < dim; i += 64) d = fmaf(RULE == 1 && bonus ? qr[at(i)] * bonus[h * dim + i] : qr[at(i)], kr[at(i)], d);      // (a lane re-reads only what it wrote itself)
             d = pi_lanes_sum<64>(d);
             if (lane == 0) dot_t[tt] = d;
         }
         __syncthreads();
         for (int tt = 0; tt < nt; tt++) {
             const float vj = vt[tt * cols + tid / R];
-            const float * kr = kt + tt * dim + sp * DPT, * qr = qt + tt * dim + sp * DPT, * gr = gt + tt * dim + sp * DPT;
-            float kk[DPT], a = 0.0f, c = 0.0f, o;
-            if (dim4) {                                                   // 16-byte LDS reads: a token costs 3 * DPT / 4 of them
+            const float * kr = kt + tt * dp + sp * (DPT + 4), * qr = qt + tt * dp + sp * (DPT + 4), * gr = gt + tt * dp + sp * (DPT + 4);
+            float a = 0.0f, c = 0.0f, o;
+            float4 k4[DPT / 4], q4[DPT / 4], g4[DPT / 4];                 // 16-byte LDS reads, no bounds (rows beyond dim: k = q = g = 0, their S stays 0): all of a token's reads go out before the first use
 #pragma unroll
-                for (int ii = 0; ii < DPT; ii += 4) {
-                    if (sp * DPT + ii < dim) {
-                        const float4 kv = *(const float4 *) (kr + ii), qv = *(const float4 *) (qr + ii), gv = *(const float4 *) (gr + ii);
-                        kk[ii] = kv.x; kk[ii + 1] = kv.y; kk[ii + 2] = kv.z; kk[ii + 3] = kv.w;
-                        if (RULE == 0) {
-                            S[ii] *= gv.x; S[ii + 1] *= gv.y; S[ii + 2] *= gv.z; S[ii + 3] *= gv.w;
-                            a = fmaf(S[ii], kv.x, a); a = fmaf(S[ii + 1], kv.y, a); a = fmaf(S[ii + 2], kv.z, a); a = fmaf(S[ii + 3], kv.w, a);
-                        }
-                        c = fmaf(S[ii], qv.x, c); c = fmaf(S[ii + 1], qv.y, c); c = fmaf(S[ii + 2], qv.z, c); c = fmaf(S[ii + 3], qv.w, c);
-                        if (RULE == 1) { S[ii] *= gv.x; S[ii + 1] *= gv.y; S[ii + 2] *= gv.z; S[ii + 3] *= gv.w; }
-                    } else { kk[ii] = kk[ii + 1] = kk[ii + 2] = kk[ii + 3] = 0.0f; }
-                }
-            } else {
+            for (int ii = 0; ii < DPT / 4; ii++) { k4[ii] = *(const float4 *) (kr + 4 * ii); q4[ii] = *(const float4 *) (qr + 4 * ii); g4[ii] = *(const float4 *) (gr + 4 * ii); }
+            float a2 = 0.0f, c2 = 0.0f;                                   // (two chains each: half the depth of the dependent sums)
 #pragma unroll
-                for (int ii = 0; ii < DPT; ii++) {
-                    if (sp * DPT + ii < dim) {
-                        kk[ii] = kr[ii];
-                        if (RULE == 0) { S[ii] *= gr[ii]; a = fmaf(S[ii], kk[ii], a); }
-                        c = fmaf(S[ii], qr[ii], c);
-                        if (RULE == 1) S[ii] *= gr[ii];
-                    } else kk[ii] = 0.0f;
+            for (int ii = 0; ii < DPT / 4; ii++) {
+                const float4 kv = k4[ii], qv = q4[ii], gv = g4[ii];
+                float * Sq = S + 4 * ii;
+                if (RULE == 0) {
+                    Sq[0] *= gv.x; Sq[1] *= gv.y; Sq[2] *= gv.z; Sq[3] *= gv.w;
+                    a = fmaf(Sq[0], kv.x, a); a2 = fmaf(Sq[1], kv.y, a2); a = fmaf(Sq[2], kv.z, a); a2 = fmaf(Sq[3], kv.w, a2);
                 }
+                c = fmaf(Sq[0], qv.x, c); c2 = fmaf(Sq[1], qv.y, c2); c = fmaf(Sq[2], qv.z, c); c2 = fmaf(Sq[3], qv.w, c2);
+                if (RULE == 1) { Sq[0] *= gv.x; Sq[1] *= gv.y; Sq[2] *= gv.z; Sq[3] *= gv.w; }
             }
+            a += a2; c += c2;
             if (R == 2) { if (RULE == 0) a += pi_partner<1>(a); c += pi_partner<1>(c); }
             else if (R == 4) { if (RULE == 0) { a += pi_partner<2>(a); a += pi_partner<1>(a); } c += pi_partner<2>(c); c += pi_partner<1>(c); }
             else for (int d = R >> 1; d > 0; d >>= 1) { if (RULE == 0) a += __shfl_xor(a, d, PI_WAVE); c += __shfl_xor(c, d, PI_WAVE); }
             const float u = RULE == 0 ? beta_t[tt] * (vj - a) : vj;       // what the token writes under its key
             o = fmaf(u, dot_t[tt], c);
 #pragma unroll
-            for (int ii = 0; ii < DPT; ii++) S[ii] = fmaf(kk[ii], u, S[ii]);
+            for (int ii = 0; ii < DPT / 4; ii++) { S[4 * ii] = fmaf(k4[ii].x, u, S[4 * ii]); S[4 * ii + 1] = fmaf(k4[ii].y, u, S[4 * ii + 1]); S[4 * ii + 2] = fmaf(k4[ii].z, u, S[4 * ii + 2]); S[4 * ii + 3] = fmaf(k4[ii].w, u, S[4 * ii + 3]); }
             if (mode != 1 && col_ok && sp == 0) out[(int64_t) (first + t0 + tt) * os + (int64_t) h * vdim + j] = o;
         }
     }
@@ -339,12 +338,13 @@ __global__ void __launch_bounds__(256) k_channel_recurrence(const float * __rest
 }
 
 // grid (head, blocks of CR_SCAN_COLS value columns, run): per piece p of the run, in order: scratch[p] holds [L_p | T_p] coming in and S_in(p) (in L_p's place) going out.
-// A workgroup keeps its columns of S in LDS (two buffers) and T_p transposed ([c][i], so that a thread's rows are neighbours); thread (column j, row part): 8 rows at a time in registers.
+// A workgroup keeps its columns of S in LDS (two buffers) and T_p transposed ([c][i], so that a thread's rows are neighbours); a thread owns a tile of 8 rows x 4 columns: per column c of T_p
+// three 16-byte LDS reads feed 32 multiply-adds.
 template <int CR_SCAN_COLS>
-__global__ void __launch_bounds__(256) k_channel_state_scan(int heads, int dim, int vdim, const float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, float * __restrict__ scratch,
-                                                            const int32_t * __restrict__ abort_w) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) k_channel_state_scan(int heads, int dim, int vdim, const float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok,
+                                                                                                     float * __restrict__ scratch, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
-    extern __shared__ float lds[];                // T^T [dim][dim + 4] | S [2][dim][CR_SCAN_COLS]
+    extern __shared__ float lds[];                // T^T [dim][tp] | S [2][dim][CR_SCAN_COLS]
     __shared__ int seg[3], bnd[CR_MAXRUNS], sorted[CR_MAXRUNS], nbnd;      // slot word, first piece ordinal, pieces of the run (0: no such run)
     const int tid = threadIdx.x, h = blockIdx.x, j0 = blockIdx.y * CR_SCAN_COLS;
     const int n_runs = cr_runs(rec, n_tok, bnd, sorted, &nbnd);
@@ -353,7 +353,7 @@ __global__ void __launch_bounds__(256) k_channel_state_scan(int heads, int dim, 
         seg[0] = -1; seg[2] = 0;
         for (int r = 0; r < n_runs; r++) {
             const int t = sorted[r], e = r + 1 < n_runs ? sorted[r + 1] : n_tok;
-            const int ns = (e - t + CR_TB - 1) / CR_TB;
+            const int ns = (e - t + CR_PIECE - 1) / CR_PIECE;
             if (r == (int) blockIdx.z) { seg[0] = rec[t]; seg[1] = ord; seg[2] = ns; break; }
             ord += ns;
         }
@@ -361,10 +361,10 @@ __global__ void __launch_bounds__(256) k_channel_state_scan(int heads, int dim, 
     __syncthreads();
     const int word = seg[0], sub0 = seg[1], nsub = seg[2];
     if (nsub == 0 || word < 0) return;
-    const int slot = word & ~CM_FRESH, sw = vdim + dim, tp = dim + 4;
+    const int slot = word & ~CM_FRESH, sw = vdim + dim, tp = (dim + 3) / 4 * 4 + 4;       // (rows of T^T start 16-byte aligned)
     float * Tt = lds, * Sb = Tt + dim * tp;
-    const int jl = tid % CR_SCAN_COLS, part = tid / CR_SCAN_COLS, j = j0 + jl, pstep = 8 * (256 / CR_SCAN_COLS);      // row parts of 8 rows
-    const bool col_ok = j < vdim;
+    constexpr int CG = CR_SCAN_COLS / 4;                               // column groups of 4
+    const int jg = tid % CG, part = tid / CG, jl = jg * 4, pstep = 8 * (256 / CG);      // row parts of 8 rows
     const float * S0 = state + ((int64_t) slot * heads + h) * dim * vdim;
     for (int idx = tid; idx < dim * CR_SCAN_COLS; idx += 256) {
         const int i = idx / CR_SCAN_COLS, jj = j0 + idx % CR_SCAN_COLS;
@@ -380,21 +380,25 @@ __global__ void __launch_bounds__(256) k_channel_state_scan(int heads, int dim, 
         const float * Sc = Sb + cur * dim * CR_SCAN_COLS;
         float * Sn = Sb + (cur ^ 1) * dim * CR_SCAN_COLS;
         for (int i0 = part * 8; i0 < dim; i0 += pstep) {
-            float acc[8];
+            float acc[8][4];
 #pragma unroll
-            for (int r = 0; r < 8; r++) acc[r] = (more && col_ok && i0 + r < dim) ? blk[(int64_t) (i0 + r) * sw + j] : 0.0f;          // L_p, read before S_in(p) takes its place
-            if (col_ok)
+            for (int r = 0; r < 8; r++)
 #pragma unroll
-                for (int r = 0; r < 8; r++) if (i0 + r < dim) blk[(int64_t) (i0 + r) * sw + j] = Sc[(i0 + r) * CR_SCAN_COLS + jl];
+                for (int u = 0; u < 4; u++) {
+                    const bool ok = i0 + r < dim && j0 + jl + u < vdim;
+                    acc[r][u] = (more && ok) ? blk[(int64_t) (i0 + r) * sw + j0 + jl + u] : 0.0f;                                     // L_p, read before S_in(p) takes its place
+                    if (ok) blk[(int64_t) (i0 + r) * sw + j0 + jl + u] = Sc[(i0 + r) * CR_SCAN_COLS + jl + u];
+                }
             if (!more) continue;
             for (int c = 0; c < dim; c++) {
-                const float sv = Sc[c * CR_SCAN_COLS + jl];
-                const float * tr = Tt + c * tp + i0;
+                const float4 sv = *(const float4 *) (Sc + c * CR_SCAN_COLS + jl);
+                const float4 ta = *(const float4 *) (Tt + c * tp + i0), tb = *(const float4 *) (Tt + c * tp + i0 + 4);      // (rows beyond dim read the pad or the next row of T^T: their sums are dropped)
+                const float tv[8] = { ta.x, ta.y, ta.z, ta.w, tb.x, tb.y, tb.z, tb.w };
 #pragma unroll
-                for (int r = 0; r < 8; r++) acc[r] = fmaf(tr[r], sv, acc[r]);      // (rows beyond dim read the pad or the next row of T^T: their sums are dropped)
+                for (int r = 0; r < 8; r++) { acc[r][0] = fmaf(tv[r], sv.x, acc[r][0]); acc[r][1] = fmaf(tv[r], sv.y, acc[r][1]); acc[r][2] = fmaf(tv[r], sv.z, acc[r][2]); acc[r][3] = fmaf(tv[r], sv.w, acc[r][3]); }
             }
 #pragma unroll
-            for (int r = 0; r < 8; r++) if (i0 + r < dim) Sn[(i0 + r) * CR_SCAN_COLS + jl] = acc[r];
+            for (int r = 0; r < 8; r++) if (i0 + r < dim) *(float4 *) (Sn + (i0 + r) * CR_SCAN_COLS + jl) = make_float4(acc[r][0], acc[r][1], acc[r][2], acc[r][3]);
         }
         cur ^= 1;
     }
@@ -412,7 +416,7 @@ __global__ void __launch_bounds__(256) k_channel_state_scan_diag(int heads, int 
         seg[0] = -1; seg[2] = 0;
         for (int r = 0; r < n_runs; r++) {
             const int t = sorted[r], e = r + 1 < n_runs ? sorted[r + 1] : n_tok;
-            const int ns = (e - t + CR_TB - 1) / CR_TB;
+            const int ns = (e - t + CR_PIECE - 1) / CR_PIECE;
             if (r == (int) blockIdx.z) { seg[0] = rec[t]; seg[1] = ord; seg[2] = ns; break; }
             ord += ns;
         }
@@ -453,10 +457,10 @@ extern "C" int pi_op_channel_recurrence_reserve(void) {
     done = true;
     return 0;
 }
-static int cr_max_pieces(int n_tok, int max_segments) { return n_tok / CR_TB + std::min(n_tok, std::max(1, max_segments)) + 1; }
+static int cr_max_pieces(int n_tok, int max_segments) { return n_tok / CR_PIECE + std::min(n_tok, std::max(1, max_segments)) + 1; }
 // passes of more than 32 tokens cut the runs into pieces that run side by side: floats of scratch they need (0: such a pass is walked in one piece per run)
 extern "C" size_t pi_op_channel_recurrence_scratch_floats(int heads, int dim, int vdim, int n_tok, int max_segments) {      // (sized for the delta rule, which needs more)
-    return (n_tok <= CR_TB || dim > CR_SCAN_MAXDIM) ? 0 : (size_t) cr_max_pieces(n_tok, max_segments) * heads * dim * (vdim + dim);
+    return (n_tok <= CR_PIECE || dim > CR_SCAN_MAXDIM) ? 0 : (size_t) cr_max_pieces(n_tok, max_segments) * heads * dim * (vdim + dim);
 }
 extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_stride, const float * k, int64_t k_stride, const float * v, int64_t v_stride, const float * decay_raw, int64_t decay_stride, int decay_mode,
                                         const float * decay_bias_dev, const float * a_log_dev, const float * beta_raw, int64_t beta_stride, const float * bonus_dev, int qk_unit, float q_mult,
@@ -481,7 +485,7 @@ extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_str
         const int threads = std::min(256, (ncol * R + 63) / 64 * 64);
         const int cols = threads / R;
         const dim3 grid((unsigned) heads, (unsigned) ((ncol + cols - 1) / cols), (unsigned) (mode ? cr_max_pieces(n_tok, max_segments) : runs));
-        const size_t lds = ((size_t) 3 * CR_TB * dim + (size_t) CR_TB * cols) * sizeof(float);
+        const size_t lds = ((size_t) 3 * CR_TB * R * (dpt + 4) + (size_t) CR_TB * cols) * sizeof(float);
         if (lds > CR_LDS_MAX) { pi_set_error("pi_op_channel_recurrence: a key width of %d needs %zu bytes of LDS (at most %d)", dim, lds, CR_LDS_MAX); return -1; }
         if (lds > 48 * 1024 && pi_op_channel_recurrence_reserve() != 0) return -1;
 #define CR_GO(D, RL) PI_KT_LAUNCH(PI_KT_ATT, 0, nta, bytes, (k_channel_recurrence<D, RL>), grid, dim3(threads), lds, s, q, q_stride, k, k_stride, v, v_stride, decay_raw, decay_stride, decay_mode, decay_bias_dev, a_log_dev, \
@@ -500,8 +504,8 @@ extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_str
     } else {
         // columns per workgroup: as few as it takes to put a workgroup on every compute unit (each one re-reads the transition matrices, which the others' reads keep in L2)
         int sc = 32;
-        while (sc > 8 && (int64_t) heads * ((vdim + sc - 1) / sc) * runs < 256) sc >>= 1;
-        const size_t scan_lds = ((size_t) dim * (dim + 4) + (size_t) 2 * dim * sc) * sizeof(float);
+        while (sc > 8 && (int64_t) heads * ((vdim + sc - 1) / sc) < 256) sc >>= 1;           // (a pass usually carries one run, whatever the slots allow)
+        const size_t scan_lds = ((size_t) dim * ((dim + 3) / 4 * 4 + 4) + (size_t) 2 * dim * sc + 8) * sizeof(float);
         if (scan_lds > 48 * 1024 && pi_op_channel_recurrence_reserve() != 0) return -1;
         const dim3 sgrid((unsigned) heads, (unsigned) ((vdim + sc - 1) / sc), (unsigned) runs);
         const double sbytes = 4.0 * n_pieces * heads * dim * (2.0 * vdim + dim);
