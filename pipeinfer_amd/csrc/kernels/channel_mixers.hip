@@ -202,13 +202,12 @@ static __device__ __forceinline__ int cr_runs(const int32_t * __restrict__ rec, 
     __syncthreads();
     return n;
 }
-// (amdgpu_waves_per_eu(1, 2): the kernel is a chain of dependent steps per token, what helps is having a token's LDS reads in flight together, which takes registers; the compiler's default
-// aims at eight waves per SIMD, keeps under 64 registers and then waits for every read on its own: 3.4 us per token, measured)
+// (amdgpu_waves_per_eu(1, 2): at most two workgroups fit a compute unit's LDS anyway, so the registers of the other waves a SIMD could hold are free for a token's reads)
 template <int DPT, int RULE>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) k_channel_recurrence(const float * __restrict__ q, int64_t qs, const float * __restrict__ k, int64_t ks, const float * __restrict__ v, int64_t vs,
                                                             const float * __restrict__ draw, int64_t ds, int decay_mode, const float * __restrict__ dbias, const float * __restrict__ a_log,
                                                             const float * __restrict__ braw, int64_t bs, const float * __restrict__ bonus, int qk_unit, float q_mult,
-                                                            int heads, int hpg, int dim, int vdim, int R, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, int mode,
+                                                            int heads, int hpg, int dim, int vdim, int R, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, int mode, int tb,
                                                             float * __restrict__ scratch, float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
     extern __shared__ float lds[];                // q [CR_TB][dp] | k [CR_TB][dp] | g [CR_TB][dp] | v [CR_TB][cols];  a row is R parts of DPT values, DPT + 4 floats apart (the parts of one wave-wide read then fall into different banks), dp = R * (DPT + 4); rows end in zeros so that the token loop needs no bounds
@@ -257,10 +256,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))
         S[ii] = s0;
     }
     const int dp = R * (DPT + 4);
-    float * qt = lds, * kt = qt + CR_TB * dp, * gt = kt + CR_TB * dp, * vt = gt + CR_TB * dp;
+    float * qt = lds, * kt = qt + tb * dp, * gt = kt + tb * dp, * vt = gt + tb * dp;        // tb <= CR_TB tokens at a time (fewer where the keys are very wide)
     const float ah = decay_mode == 2 ? expf(a_log[h]) : 0.0f;
-    for (int t0 = 0; t0 < len; t0 += CR_TB) {
-        const int nt = min(CR_TB, len - t0);
+    for (int t0 = 0; t0 < len; t0 += tb) {
+        const int nt = min(tb, len - t0);
         __syncthreads();
         for (int idx = tid; idx < nt * R * DPT; idx += blockDim.x) {
             const int tt = idx / (R * DPT), i = idx % (R * DPT);
@@ -485,11 +484,14 @@ extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_str
         const int threads = std::min(256, (ncol * R + 63) / 64 * 64);
         const int cols = threads / R;
         const dim3 grid((unsigned) heads, (unsigned) ((ncol + cols - 1) / cols), (unsigned) (mode ? cr_max_pieces(n_tok, max_segments) : runs));
-        const size_t lds = ((size_t) 3 * CR_TB * R * (dpt + 4) + (size_t) CR_TB * cols) * sizeof(float);
+        int tb = CR_TB;                                                 // tokens staged at a time: as many as the LDS takes
+        auto lds_of = [&](int n) { return ((size_t) 3 * n * R * (dpt + 4) + (size_t) n * cols) * sizeof(float); };
+        while (tb > 1 && lds_of(tb) > CR_LDS_MAX) tb >>= 1;
+        const size_t lds = lds_of(tb);
         if (lds > CR_LDS_MAX) { pi_set_error("pi_op_channel_recurrence: a key width of %d needs %zu bytes of LDS (at most %d)", dim, lds, CR_LDS_MAX); return -1; }
         if (lds > 48 * 1024 && pi_op_channel_recurrence_reserve() != 0) return -1;
 #define CR_GO(D, RL) PI_KT_LAUNCH(PI_KT_ATT, 0, nta, bytes, (k_channel_recurrence<D, RL>), grid, dim3(threads), lds, s, q, q_stride, k, k_stride, v, v_stride, decay_raw, decay_stride, decay_mode, decay_bias_dev, a_log_dev, \
-                                  beta_raw, beta_stride, bonus_dev, qk_unit, q_mult, heads, heads / qk_heads, dim, vdim, R, state_dev, rec_dev, n_tok, mode, scratch_dev, out, out_stride, pi_abort_word())
+                                  beta_raw, beta_stride, bonus_dev, qk_unit, q_mult, heads, heads / qk_heads, dim, vdim, R, state_dev, rec_dev, n_tok, mode, tb, scratch_dev, out, out_stride, pi_abort_word())
         if (rule == PI_RULE_DELTA) { if (dpt == 8) CR_GO(8, 0); else if (dpt == 16) CR_GO(16, 0); else CR_GO(32, 0); }
         else                       { if (dpt == 8) CR_GO(8, 1); else if (dpt == 16) CR_GO(16, 1); else CR_GO(32, 1); }
 #undef CR_GO

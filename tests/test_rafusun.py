@@ -306,7 +306,7 @@ def recurrence_ref(rule, q, k, v, g, beta, bonus, S):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("H,G,D,V", [(2, 1, 6, 5), (1, 1, 40, 70), (4, 2, 33, 8), (3, 3, 130, 20), (2, 2, 8, 300), (1, 1, 1, 1)])
+@pytest.mark.parametrize("H,G,D,V", [(2, 1, 6, 5), (1, 1, 40, 70), (4, 2, 33, 8), (3, 3, 130, 20), (2, 2, 8, 300), (1, 1, 1, 1), (1, 1, 600, 12)])
 @pytest.mark.parametrize("rule", [DELTA, BONUS])
 @pytest.mark.parametrize("pieces", [False, True])
 def test_channel_recurrence_rules_decays_and_passes(H, G, D, V, rule, pieces):
