@@ -438,16 +438,20 @@ static bool forward_post_norm_blocks(llama_context * ctx, int n_tok, int n_kv) {
         if (H.mixer == PI_MIXER_CHANNEL_DELTA) {
             const pi_channel_delta & D = H.delta;
             const int64_t pw = D.in_rows(), gd = (int64_t) D.kv_heads * D.dim, hd = (int64_t) D.heads * D.dim, hv = (int64_t) D.heads * D.vdim, ch = D.channels();
-            float * C = A, * A2 = C + (size_t) nb * ch, * G2 = A2 + (size_t) nb * hd, * O = G2 + (size_t) nb * hv;
+            const int64_t aw = hd + hv;                                                                // a token's row of [raw decays | raw gate]
+            float * C = A, * A2 = C + (size_t) nb * ch, * G2 = A2 + hd, * O = A2 + (size_t) nb * aw;
             float * S = ctx->rec_state + ctx->rec_off[il], * conv_state = S + (size_t) n_slots * D.matrix_floats();
             OP_OK(pi_op_dense(W.w_in, x, width, n_tok, P, pw, PI_ACT_NONE, pw, PI_ACT_NONE, ex, s));
             OP_OK(pi_op_causal_conv(P, pw, (int) ch, D.conv, W.conv_w, nullptr, conv_state, ctx->rec_dev, n_tok, PI_ACT_SILU, C, ch, s));
-            OP_OK(pi_op_dense(W.w_a2, P + ch, pw, n_tok, A2, hd, PI_ACT_NONE, hd, PI_ACT_NONE, ex, s));
-            OP_OK(pi_op_dense(W.w_g2, P + ch + D.decay_rank, pw, n_tok, G2, hv, PI_ACT_NONE, hv, PI_ACT_NONE, ex, s));
-            OP_OK(pi_op_channel_recurrence(PI_RULE_DELTA, C, ch, C + gd, ch, C + 2 * gd, ch, A2, hd, 2, W.dt_bias, W.a_log, P + ch + D.decay_rank + D.gate_rank, pw, nullptr, 1, 1.0f / sqrtf((float) D.dim), D.heads, D.kv_heads, D.dim, D.vdim,
+            if (!W.w_g2) OP_OK(pi_op_dense_segments(W.w_a2, P + ch, pw, hd, D.decay_rank, 2, n_tok, A2, aw, PI_ACT_NONE, aw, PI_ACT_NONE, ex, s));
+            else {
+                OP_OK(pi_op_dense(W.w_a2, P + ch, pw, n_tok, A2, aw, PI_ACT_NONE, hd, PI_ACT_NONE, ex, s));
+                OP_OK(pi_op_dense(W.w_g2, P + ch + D.decay_rank, pw, n_tok, G2, aw, PI_ACT_NONE, hv, PI_ACT_NONE, ex, s));
+            }
+            OP_OK(pi_op_channel_recurrence(PI_RULE_DELTA, C, ch, C + gd, ch, C + 2 * gd, ch, A2, aw, 2, W.dt_bias, W.a_log, P + ch + D.decay_rank + D.gate_rank, pw, nullptr, 1, 1.0f / sqrtf((float) D.dim), D.heads, D.kv_heads, D.dim, D.vdim,
                                            S, ctx->rec_dev, n_tok, n_slots, ctx->rec_scratch, ctx->rec_scratch_floats, O, hv, s));
             trace(ctx, "rec", (int) il, O, hv, n_tok);
-            OP_OK(pi_op_head_norm_gate(O, hv, D.heads, D.vdim, W.mix_norm, 0, G2, hv, PI_ACT_SIGMOID, eps, n_tok, O, hv, s));
+            OP_OK(pi_op_head_norm_gate(O, hv, D.heads, D.vdim, W.mix_norm, 0, G2, aw, PI_ACT_SIGMOID, eps, n_tok, O, hv, s));
             OP_OK(pi_op_dense(W.w_o, O, hv, n_tok, Y, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
         } else if (H.mixer == PI_MIXER_PARALLEL_SHIFT) {
             const pi_gate_attention & L = H.left; const pi_time_mix & R = H.shift;

@@ -280,7 +280,10 @@ bool llama_model::ensure_loaded_hybrid(int n_positions, std::string & err) {
                 const std::string m = p + "mix.";
                 const int64_t gd = (int64_t) D.kv_heads * D.dim, hd = (int64_t) D.heads * D.dim, hv = (int64_t) D.heads * D.vdim;
                 if (!(W.w_in = L.matrix({ { m + "q", gd }, { m + "k", gd }, { m + "v", hv }, { m + "a1", D.decay_rank }, { m + "g1", D.gate_rank }, { m + "b", D.heads } }, width))) return false;
-                if (!(W.w_a2 = L.matrix({ { m + "a2", hd } }, D.decay_rank)) || !(W.w_g2 = L.matrix({ { m + "g2", hv } }, D.gate_rank)) || !(W.w_o = L.matrix({ { m + "o", width } }, hv))) return false;
+                // the second halves of the two low-rank projections: one matrix [a2 | g2] in two segments where their ranks are equal (one launch), two matrices otherwise
+                if (D.decay_rank == D.gate_rank) { if (!(W.w_a2 = L.matrix({ { m + "a2", hd }, { m + "g2", hv } }, D.decay_rank))) return false; }
+                else if (!(W.w_a2 = L.matrix({ { m + "a2", hd } }, D.decay_rank)) || !(W.w_g2 = L.matrix({ { m + "g2", hv } }, D.gate_rank))) return false;
+                if (!(W.w_o = L.matrix({ { m + "o", width } }, hv))) return false;
                 if (!(W.conv_w = L.vectors({ { m + "q.conv", gd }, { m + "k.conv", gd }, { m + "v.conv", hv } }, D.conv))) return false;
                 if (!(W.a_log = L.vector(m + "A_log", D.heads)) || !(W.dt_bias = L.vector(m + "dt_bias", hd)) || !(W.mix_norm = L.vector(m + "norm", D.vdim))) return false;
             } else if (H.mixer == PI_MIXER_PARALLEL_SHIFT) {

@@ -394,12 +394,16 @@ __global__ void __launch_bounds__(256) k_conv_state_update(const float * __restr
     }
 }
 
+static bool pi_causal_conv_walk_ok(int n_tok, int taps);
+static int pi_causal_conv_walk(const float * x, int64_t x_stride, int channels, int taps, const float * w_dev, const float * bias_dev, float * state_dev, const int32_t * rec_dev, int n_tok, int act, float * out,
+                               int64_t out_stride, hipStream_t s);
 extern "C" int pi_op_causal_conv(const float * x, int64_t x_stride, int channels, int taps, const float * w_dev, const float * bias_dev, float * state_dev, const int32_t * rec_dev, int n_tok, int act,
                                  float * out, int64_t out_stride, void * stream) {
     if (n_tok <= 0 || channels <= 0) return 0;
     if (taps < 1 || taps > 64) { pi_set_error("pi_op_causal_conv: %d taps (1..64)", taps); return -1; }
     if (out == x) { pi_set_error("pi_op_causal_conv: the output may not overwrite the input (later tokens and the state read it)"); return -1; }
     hipStream_t s = (hipStream_t) stream;
+    if (pi_causal_conv_walk_ok(n_tok, taps)) return pi_causal_conv_walk(x, x_stride, channels, taps, w_dev, bias_dev, state_dev, rec_dev, n_tok, act, out, out_stride, s);      // short passes: one launch, the state included
     const dim3 grid((unsigned) n_tok, (unsigned) ((channels + 255) / 256));
     PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 8.0 * n_tok * channels + 4.0 * channels * taps, k_causal_conv, grid, dim3(256), 0, s, x, x_stride, channels, taps, w_dev, bias_dev, state_dev, rec_dev, act, out, out_stride, pi_abort_word());
     PI_CHECK_LAUNCH();
@@ -455,6 +459,16 @@ __global__ void __launch_bounds__(256) k_causal_conv_walk(const float * __restri
     for (int l = 0; l < CV_MAXTAPS - 1; l++) if (l >= off) st[(int64_t) (l - off) * channels] = win[l];
 }
 #define CV_WALK_MAX_TOKENS 32
+static bool pi_causal_conv_walk_ok(int n_tok, int taps) { return n_tok <= CV_WALK_MAX_TOKENS && taps <= CV_MAXTAPS; }
+// the walking kernel without the row of blocks that forms step sizes
+static int pi_causal_conv_walk(const float * x, int64_t x_stride, int channels, int taps, const float * w_dev, const float * bias_dev, float * state_dev, const int32_t * rec_dev, int n_tok, int act, float * out,
+                               int64_t out_stride, hipStream_t s) {
+    const int cblocks = (channels + 255) / 256;
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 8.0 * n_tok * channels + 4.0 * channels * (2 * taps - 1), k_causal_conv_walk, dim3((unsigned) n_tok, (unsigned) cblocks), dim3(256), 0, s,
+                 x, x_stride, channels, taps, w_dev, bias_dev, state_dev, rec_dev, n_tok, act, out, out_stride, cblocks, (const float *) nullptr, (int64_t) 0, (const float *) nullptr, (const float *) nullptr, 0,
+                 (float *) nullptr, (float *) nullptr, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
 // the convolution and, in the same launch where the pass is short, the step sizes / decays of the recurrence it feeds (raw_dev .. decay_out as for pi_op_ssd_steps)
 extern "C" int pi_op_causal_conv_steps(const float * x, int64_t x_stride, int channels, int taps, const float * w_dev, const float * bias_dev, float * state_dev, const int32_t * rec_dev, int n_tok, int act,
                                        float * out, int64_t out_stride, const float * raw, int64_t raw_stride, const float * dt_bias_dev, const float * a_log_dev, int heads, float * dt_out, float * decay_out,
