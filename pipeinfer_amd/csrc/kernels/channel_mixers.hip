@@ -183,7 +183,7 @@ extern "C" int pi_op_token_shift(const float * h, int64_t h_stride, int n, const
 //   k_channel_state_scan / _diag  per run, piece by piece: S_in(p + 1) = T_p S_in(p) + L_p, S_in(0) = the slot's state (or zero); scratch[p][..][0 .. vdim) <- S_in(p)
 //   mode 2  every piece from its true S_in(p): outputs; a run's last piece leaves the slot's new state
 #define CR_TB 32                                  // tokens staged in LDS at a time
-#define CR_PIECE 64                               // tokens of a piece of a long pass (two tiles: half the pieces for the scan to chain, the same LDS)
+#define CR_PIECE 64                               // most tokens of a piece of a long pass (the launcher picks 32 or 64: longer pieces leave the scan fewer to chain, shorter ones put more side by side)
 #define CR_MAXRUNS 256
 #define CR_SCAN_MAXDIM 128                        // widest key whose transition matrix the scan keeps in LDS
 // the pass's runs in order (a run: the consecutive tokens of one slot): every thread looks at its own tokens for a run's first one, the few found are ranked by position.  first[r] in `sorted`
@@ -207,7 +207,7 @@ template <int DPT, int RULE>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))) k_channel_recurrence(const float * __restrict__ q, int64_t qs, const float * __restrict__ k, int64_t ks, const float * __restrict__ v, int64_t vs,
                                                             const float * __restrict__ draw, int64_t ds, int decay_mode, const float * __restrict__ dbias, const float * __restrict__ a_log,
                                                             const float * __restrict__ braw, int64_t bs, const float * __restrict__ bonus, int qk_unit, float q_mult,
-                                                            int heads, int hpg, int dim, int vdim, int R, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, int mode, int tb,
+                                                            int heads, int hpg, int dim, int vdim, int R, float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, int mode, int tb, int piece,
                                                             float * __restrict__ scratch, float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
     extern __shared__ float lds[];                // q [CR_TB][dp] | k [CR_TB][dp] | g [CR_TB][dp] | v [CR_TB][cols];  a row is R parts of DPT values, DPT + 4 floats apart (the parts of one wave-wide read then fall into different banks), dp = R * (DPT + 4); rows end in zeros so that the token loop needs no bounds
@@ -217,7 +217,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))
     const int n_runs = n_tok == 1 ? 1 : cr_runs(rec, n_tok, bnd, sorted, &nbnd);      // (a single token is its own run: no search, no barrier)
     if (n_tok == 1) { if (tid == 0) { seg[0] = 0; seg[1] = blockIdx.z == 0 ? 1 : 0; seg[2] = rec[0]; seg[3] = 1; } }
     else if (tid == 0) {                          // piece number blockIdx.z of the pass (mode 0: pieces are whole runs)
-        const int lseg = mode ? CR_PIECE : 0, want = blockIdx.z;
+        const int lseg = mode ? piece : 0, want = blockIdx.z;
         int ord = 0;
         seg[1] = 0; seg[2] = -1;
         for (int r = 0; r < n_runs; r++) {
@@ -340,7 +340,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 2))
 // A workgroup keeps its columns of S in LDS (two buffers) and T_p transposed ([c][i], so that a thread's rows are neighbours); a thread owns a tile of 8 rows x 4 columns: per column c of T_p
 // three 16-byte LDS reads feed 32 multiply-adds.
 template <int CR_SCAN_COLS>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) k_channel_state_scan(int heads, int dim, int vdim, const float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok,
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))) k_channel_state_scan(int heads, int dim, int vdim, int piece, const float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok,
                                                                                                      float * __restrict__ scratch, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
     extern __shared__ float lds[];                // T^T [dim][tp] | S [2][dim][CR_SCAN_COLS]
@@ -352,7 +352,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))
         seg[0] = -1; seg[2] = 0;
         for (int r = 0; r < n_runs; r++) {
             const int t = sorted[r], e = r + 1 < n_runs ? sorted[r + 1] : n_tok;
-            const int ns = (e - t + CR_PIECE - 1) / CR_PIECE;
+            const int ns = (e - t + piece - 1) / piece;
             if (r == (int) blockIdx.z) { seg[0] = rec[t]; seg[1] = ord; seg[2] = ns; break; }
             ord += ns;
         }
@@ -404,7 +404,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 4))
 }
 
 // the same chain where T_p is diagonal (bonus rule): scratch[p] holds [L_p | diag T_p] ([dim][vdim + 1]).  grid (head, blocks over dim * vdim, run): eight pieces' loads in flight, the chain in registers
-__global__ void __launch_bounds__(256) k_channel_state_scan_diag(int heads, int dim, int vdim, const float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, float * __restrict__ scratch,
+__global__ void __launch_bounds__(256) k_channel_state_scan_diag(int heads, int dim, int vdim, int piece, const float * __restrict__ state, const int32_t * __restrict__ rec, int n_tok, float * __restrict__ scratch,
                                                                  const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
     __shared__ int seg[3], bnd[CR_MAXRUNS], sorted[CR_MAXRUNS], nbnd;
@@ -415,7 +415,7 @@ __global__ void __launch_bounds__(256) k_channel_state_scan_diag(int heads, int 
         seg[0] = -1; seg[2] = 0;
         for (int r = 0; r < n_runs; r++) {
             const int t = sorted[r], e = r + 1 < n_runs ? sorted[r + 1] : n_tok;
-            const int ns = (e - t + CR_PIECE - 1) / CR_PIECE;
+            const int ns = (e - t + piece - 1) / piece;
             if (r == (int) blockIdx.z) { seg[0] = rec[t]; seg[1] = ord; seg[2] = ns; break; }
             ord += ns;
         }
@@ -456,10 +456,10 @@ extern "C" int pi_op_channel_recurrence_reserve(void) {
     done = true;
     return 0;
 }
-static int cr_max_pieces(int n_tok, int max_segments) { return n_tok / CR_PIECE + std::min(n_tok, std::max(1, max_segments)) + 1; }
+static int cr_max_pieces(int n_tok, int max_segments, int piece = CR_TB) { return n_tok / piece + std::min(n_tok, std::max(1, max_segments)) + 1; }
 // passes of more than 32 tokens cut the runs into pieces that run side by side: floats of scratch they need (0: such a pass is walked in one piece per run)
 extern "C" size_t pi_op_channel_recurrence_scratch_floats(int heads, int dim, int vdim, int n_tok, int max_segments) {      // (sized for the delta rule, which needs more)
-    return (n_tok <= CR_PIECE || dim > CR_SCAN_MAXDIM) ? 0 : (size_t) cr_max_pieces(n_tok, max_segments) * heads * dim * (vdim + dim);
+    return (n_tok <= CR_TB || dim > CR_SCAN_MAXDIM) ? 0 : (size_t) cr_max_pieces(n_tok, max_segments) * heads * dim * (vdim + dim);
 }
 extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_stride, const float * k, int64_t k_stride, const float * v, int64_t v_stride, const float * decay_raw, int64_t decay_stride, int decay_mode,
                                         const float * decay_bias_dev, const float * a_log_dev, const float * beta_raw, int64_t beta_stride, const float * bonus_dev, int qk_unit, float q_mult,
@@ -479,11 +479,14 @@ extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_str
     const double bytes = 4.0 * n_tok * heads * (3.0 * dim + 2.0 * vdim) + 8.0 * heads * dim * vdim;
     hipStream_t s = (hipStream_t) stream;
     const int nta = std::min(n_tok, PI_KT_MAXNT - 1);
+    // delta rule: the scan's work grows with the number of pieces, so pieces of 64 tokens where that still leaves a workgroup per compute unit; bonus rule (a scan of no weight): 32
+    const int cols0 = std::min(256, (vdim * R + 63) / 64 * 64) / R;
+    const int piece = (rule == PI_RULE_DELTA && (int64_t) heads * ((vdim + cols0 - 1) / cols0) * (n_tok / CR_PIECE) >= 256) ? CR_PIECE : CR_TB;
     auto launch = [&](int mode) -> int {
         const int ncol = mode == 1 ? vdim + (rule == PI_RULE_DELTA ? dim : 1) : vdim;
         const int threads = std::min(256, (ncol * R + 63) / 64 * 64);
         const int cols = threads / R;
-        const dim3 grid((unsigned) heads, (unsigned) ((ncol + cols - 1) / cols), (unsigned) (mode ? cr_max_pieces(n_tok, max_segments) : runs));
+        const dim3 grid((unsigned) heads, (unsigned) ((ncol + cols - 1) / cols), (unsigned) (mode ? cr_max_pieces(n_tok, max_segments, piece) : runs));
         int tb = CR_TB;                                                 // tokens staged at a time: as many as the LDS takes
         auto lds_of = [&](int n) { return ((size_t) 3 * n * R * (dpt + 4) + (size_t) n * cols) * sizeof(float); };
         while (tb > 1 && lds_of(tb) > CR_LDS_MAX) tb >>= 1;
@@ -491,7 +494,7 @@ extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_str
         if (lds > CR_LDS_MAX) { pi_set_error("pi_op_channel_recurrence: a key width of %d needs %zu bytes of LDS (at most %d)", dim, lds, CR_LDS_MAX); return -1; }
         if (lds > 48 * 1024 && pi_op_channel_recurrence_reserve() != 0) return -1;
 #define CR_GO(D, RL) PI_KT_LAUNCH(PI_KT_ATT, 0, nta, bytes, (k_channel_recurrence<D, RL>), grid, dim3(threads), lds, s, q, q_stride, k, k_stride, v, v_stride, decay_raw, decay_stride, decay_mode, decay_bias_dev, a_log_dev, \
-                                  beta_raw, beta_stride, bonus_dev, qk_unit, q_mult, heads, heads / qk_heads, dim, vdim, R, state_dev, rec_dev, n_tok, mode, tb, scratch_dev, out, out_stride, pi_abort_word())
+                                  beta_raw, beta_stride, bonus_dev, qk_unit, q_mult, heads, heads / qk_heads, dim, vdim, R, state_dev, rec_dev, n_tok, mode, tb, piece, scratch_dev, out, out_stride, pi_abort_word())
         if (rule == PI_RULE_DELTA) { if (dpt == 8) CR_GO(8, 0); else if (dpt == 16) CR_GO(16, 0); else CR_GO(32, 0); }
         else                       { if (dpt == 8) CR_GO(8, 1); else if (dpt == 16) CR_GO(16, 1); else CR_GO(32, 1); }
 #undef CR_GO
@@ -499,10 +502,10 @@ extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_str
     };
     if (!pieces) return launch(0);
     if (launch(1) != 0) return -1;
-    const int n_pieces = cr_max_pieces(n_tok, max_segments);
+    const int n_pieces = cr_max_pieces(n_tok, max_segments, piece);
     if (rule == PI_RULE_BONUS) {
         PI_KT_LAUNCH(PI_KT_ATT, 0, nta, 12.0 * n_pieces * heads * dim * vdim, k_channel_state_scan_diag, dim3((unsigned) heads, (unsigned) (((int64_t) dim * vdim + 255) / 256), (unsigned) runs), dim3(256), 0, s,
-                     heads, dim, vdim, state_dev, rec_dev, n_tok, scratch_dev, pi_abort_word());
+                     heads, dim, vdim, piece, state_dev, rec_dev, n_tok, scratch_dev, pi_abort_word());
     } else {
         // columns per workgroup: as few as it takes to put a workgroup on every compute unit (each one re-reads the transition matrices, which the others' reads keep in L2)
         int sc = 32;
@@ -511,7 +514,7 @@ extern "C" int pi_op_channel_recurrence(int rule, const float * q, int64_t q_str
         if (scan_lds > 48 * 1024 && pi_op_channel_recurrence_reserve() != 0) return -1;
         const dim3 sgrid((unsigned) heads, (unsigned) ((vdim + sc - 1) / sc), (unsigned) runs);
         const double sbytes = 4.0 * n_pieces * heads * dim * (2.0 * vdim + dim);
-#define CR_SCAN(C) PI_KT_LAUNCH(PI_KT_ATT, 0, nta, sbytes, k_channel_state_scan<C>, sgrid, dim3(256), scan_lds, s, heads, dim, vdim, state_dev, rec_dev, n_tok, scratch_dev, pi_abort_word())
+#define CR_SCAN(C) PI_KT_LAUNCH(PI_KT_ATT, 0, nta, sbytes, k_channel_state_scan<C>, sgrid, dim3(256), scan_lds, s, heads, dim, vdim, piece, state_dev, rec_dev, n_tok, scratch_dev, pi_abort_word())
         if (sc == 8) CR_SCAN(8); else if (sc == 16) CR_SCAN(16); else CR_SCAN(32);
 #undef CR_SCAN
     }
