@@ -177,7 +177,8 @@ PI_API int pi_op_topk(const float * logits_dev, int n_vocab, int n_tok, int k, i
 /* ---- dense bfloat16 matrices and the operators of hybrid blocks (recurrent / low-rank-attention mixers, routed feed-forwards) --------------------------------------
  * Weights are PI_BF16 pi_weights ([rows][K] as stored, pi_weight_upload(PI_BF16, K, rows, ...)); activations, norms, scores, states and outputs are fp32.
  * exact = 0: activations are rounded to bfloat16 where they enter a matrix product (fp32 accumulation); exact = 1: nothing is rounded, every product is an fp32 fma. */
-enum pi_act { PI_ACT_NONE = 0, PI_ACT_SILU = 1, PI_ACT_SIGMOID = 2, PI_ACT_RELU_SQR = 3, PI_ACT_TANH = 4, PI_ACT_GELU_TANH = 5 /* 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))) */ };
+enum pi_act { PI_ACT_NONE = 0, PI_ACT_SILU = 1, PI_ACT_SIGMOID = 2, PI_ACT_RELU_SQR = 3, PI_ACT_TANH = 4, PI_ACT_GELU_TANH = 5 /* 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))) */,
+              PI_ACT_GELU_ERF = 6 /* 0.5 z (1 + erf(z / sqrt 2)) */ };
 /* out[t][:] = widen(table[tokens[t]]) * scale */
 PI_API int pi_op_embed(const pi_weight * table, const int32_t * tokens_dev, int n_tok, float scale, float * out_dev, void * stream);
 /* out[t][r] = act(W[r] . x[t]); rows [0, rows_a) take act_a, the others act_b (projections that share their input are one matrix and one launch); strides in floats */
@@ -318,6 +319,44 @@ enum pi_attention_weights { PI_WEIGHTS_SIGMOID = 0, PI_WEIGHTS_SOFTMAX = 1, PI_W
 PI_API int pi_op_chunk_attention_ex(const float * q_dev, int64_t q_stride, const float * k_cache_dev, const float * v_cache_dev, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
                                     const float * head_bias_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int weights, float softcap, int chunk, int heads, int kv_heads,
                                     int dim, int vdim, int n_tok, int n_kv, float * out_dev, int64_t out_stride, const int32_t * dyn_dev, void * stream);
+
+/* ---- operators of layers whose mixer and feed-forward read ONE tanh norm, of sliding-window attention with pooled far blocks, and of clipped gated experts ------------------- */
+/* rows of n floats, strides in floats */
+PI_API int pi_op_copy_rows(const float * src_dev, int64_t src_stride, float * dst_dev, int64_t dst_stride, int n, int n_tok, void * stream);
+/* the end of a layer and the norm of what reads the stream next, in one launch:  x_out = x + a + b + c (a, b, c nullable; x_out may be x);  w != NULL: h_out = tanh(alpha * x_out) * w + bias
+ * (a norm without statistics; alpha_dev: one float on the device).  x_out may be NULL when only the norm is wanted (then a, b, c are still added for h) */
+PI_API int pi_op_sum_tanh_norm(const float * x_dev, int64_t x_stride, const float * a_dev, int64_t a_stride, const float * b_dev, int64_t b_stride, const float * c_dev, int64_t c_stride, int n, int n_tok,
+                               float * x_out_dev, int64_t x_out_stride, const float * alpha_dev, const float * w_dev, const float * bias_dev, float * h_out_dev, int64_t h_out_stride, void * stream);
+/* pi_rotary_table_create with angle steps stretched by wavelength l = 2 pi / f against `original` positions: f stays where l < original / high, becomes f / factor where l > original / low, and
+ * (1 - s) f / factor + s f with s = (original / l - low) / (high - low) between the two */
+PI_API void * pi_rotary_table_create_scaled(int n_pos, int dims, float base, float factor, float low, float high, int original);
+/* pi_op_qkv_prepare_ex's norm_first takes these: rotation first, then R(.) * w over the rotated head; R(.) * w, then the rotation; the rotation alone */
+enum pi_qk_norm { PI_QK_NORM_LAST = 0, PI_QK_NORM_FIRST = 1, PI_QK_NORM_NONE = 2 };
+/* which cells of its sequence a token sees besides "not later": those of its own block of `size` positions (blocks start at multiples of size), or the last `size` positions up to itself */
+enum pi_mask_kind { PI_MASK_CHUNK = 0, PI_MASK_WINDOW = 1 };
+/* Pooled far blocks.  The caches hold two rows per cell: row c the token's own key / value, row pooled_row_offset + c — on the cell of a block's LAST position, (pos + 1) % pool == 0 — the means of the
+ * keys / values of the block's `pool` positions as the cache holds them, summed in position order.  This writes those rows for the tokens of the pass that complete a block (their block mates are the
+ * visible cells of the `pool - 1` positions before them); call it behind pi_op_qkv_prepare(_ex) and ahead of the attention.  k_cache: [2 * offset.. rows][kv_heads * dim], v_cache likewise */
+PI_API int pi_op_pool_blocks(float * k_cache_dev, float * v_cache_dev, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev, int pool, int64_t pooled_row_offset, int kv_heads, int dim, int vdim,
+                             int n_tok, int n_kv, const int32_t * dyn_dev, void * stream);
+/* pi_op_chunk_attention_ex with the mask kind as a parameter and two more sources of weight.  mask_kind PI_MASK_WINDOW: a token at position p sees the cells of its sequence at positions (p - size, p]
+ * (size 0: all up to p); pool > 0 (windows only): and for every block of `pool` positions that ends at or before p - size the pooled row (pi_op_pool_blocks) of the block's last cell, in the same soft-max.
+ * sink_dev (nullable, fp32 [heads]; soft-max kinds): exp(sink[h]) joins the denominator, without a value and without the scale (PI_WEIGHTS_SOFTMAX_SINK alone is sink = 0) */
+PI_API int pi_op_window_attention(const float * q_dev, int64_t q_stride, const float * k_cache_dev, const float * v_cache_dev, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
+                                  const float * head_bias_dev, const float * sink_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int weights, float softcap, int mask_kind, int size,
+                                  int pool, int64_t pooled_row_offset, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv, float * out_dev, int64_t out_stride, const int32_t * dyn_dev, void * stream);
+/* router by logits: z = W x + bias (bias nullable), the `top` largest z win (lowest index on a tie), their weights are the soft-max over the chosen z alone */
+PI_API int pi_op_moe_route_top_logits(const pi_weight * router, const float * bias_dev, const float * x_dev, int64_t x_stride, int n_tok, int top, int exact, int32_t * sel_dev, float * selw_dev, void * stream);
+/* the expert operators with one more kind of hidden layer.  PI_GLU_OFF / PI_GLU_SILU are glu = 0 / 1 of pi_op_moe_experts_act; PI_GLU_CLIPPED: g = min(gate, limit), u = clip(up, -limit, limit)
+ * (limit <= 0: no bounds), hidden = g * sigmoid(1.702 g) * (u + 1) */
+enum pi_glu_kind { PI_GLU_OFF = 0, PI_GLU_SILU = 1, PI_GLU_CLIPPED = 2 };
+PI_API int pi_op_moe_experts_glu(const pi_weight * w_up, const pi_weight * w_down, int n_exp, int ff, int glu, float limit, const float * x_dev, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok,
+                                 int top, int exact, float * up_dev, float * out_dev, int64_t out_stride, void * stream);
+PI_API int pi_op_moe_experts_grouped_glu(const pi_weight * w_up, const pi_weight * w_down, int n_exp, int ff, int glu, float limit, const float * x_dev, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev,
+                                         int n_tok, int top, float * up_dev, float * dn_dev, int32_t * idx_dev, float * out_dev, int64_t out_stride, void * stream);
+/* out[t][f] = hidden(in[t][f], in[t][ff + f]) [* sigmoid(in[t][gate_col])]: a gated hidden layer whose halves [gate | up] a projection left raw (glu / limit as above, PI_GLU_OFF: the plain product of
+ * pi_op_glu_mul); gate_col >= 0: one more column of the same rows holds a per-token gate */
+PI_API int pi_op_glu_mul_ex(const float * in_dev, int64_t in_stride, int ff, int glu, float limit, int64_t gate_col, int n_tok, float * out_dev, int64_t out_stride, void * stream);
 
 #ifdef __cplusplus
 }

@@ -34,7 +34,9 @@
 enum pi_arch { PI_ARCH_LLAMA = 0, PI_ARCH_FALCON = 1, PI_ARCH_BAICHUAN = 2, PI_ARCH_STARCODER = 3, PI_ARCH_REFACT = 4, PI_ARCH_BLOOM = 5, PI_ARCH_MPT = 6, PI_ARCH_STABLELM = 7, PI_ARCH_PERSIMMON = 8,
                PI_ARCH_FASOVIK = 9 /* a hybrid model: a list of layers, each with its own mixer (pi_hybrid_layer), read from config.json + model.safetensors */,
                PI_ARCH_VIKARAX = 10 /* hybrid as well: layer norms before and after every sublayer, a learned average over depth, mixers of two parallel branches */,
-               PI_ARCH_RAFUSUN = 11 /* hybrid as well: the norm AFTER the sum (x <- R(alpha x + ls * sublayer(x)) * w), a hashed pair embedding, delta-rule and attention + time-mix mixers */ };
+               PI_ARCH_RAFUSUN = 11 /* hybrid as well: the norm AFTER the sum (x <- R(alpha x + ls * sublayer(x)) * w), a hashed pair embedding, delta-rule and attention + time-mix mixers */,
+               PI_ARCH_RAREVIK = 12 /* hybrid as well: ONE tanh norm per layer that mixer and feed-forward both read (x <- x + mixer(shift(h)) + ff(h)), a run of layers repeated with the same tensors,
+                                       sliding-window attention with pooled far blocks and a learned sink, or with a per-head output gate; clipped gated experts behind a top-logit router */ };
 
 // what the reference's build_* functions differ in (llama.cpp:3985-4104 baichuan, 4229-4327 starcoder, 4540-4630 refact, 4632-4725 bloom, 4727-4825 mpt, 4827-4939 stablelm)
 struct pi_block {
@@ -54,11 +56,21 @@ enum pi_mixer_kind { PI_MIXER_LATENT_ATTENTION = 0,   // keys / values are up-pr
                      PI_MIXER_LIGHTNING = 1,          // linear attention with a per-head decay: a [dim][vdim] state per head and sequence
                      PI_MIXER_PARALLEL = 2,           // two branches that read the same input, summed with fixed factors: chunked sigmoid attention (pi_gate_attention) + a selective recurrence (pi_ssd)
                      PI_MIXER_CHANNEL_DELTA = 3,      // gated delta rule with a decay per key channel behind short convolutions (pi_channel_delta)
-                     PI_MIXER_PARALLEL_SHIFT = 4 };   // two branches, each RMS-normed over the width, averaged: chunked soft-max attention (pi_gate_attention) + time mixing with a token shift (pi_time_mix)
+                     PI_MIXER_PARALLEL_SHIFT = 4,     // two branches, each RMS-normed over the width, averaged: chunked soft-max attention (pi_gate_attention) + time mixing with a token shift (pi_time_mix)
+                     PI_MIXER_WINDOW_ATTENTION = 5 }; // soft-max attention over a sliding window of positions (pi_gate_attention with mask_kind = PI_MASK_WINDOW), optionally: a short convolution behind the projections, one pooled
+                                                      // key / value per block of positions that has left the window, a learned sink, a per-head sigmoid gate; reads the layer's token-shifted input
 // attention with grouped key / value heads, normed and partly rotated q / k, unit-norm values, un-normalised sigmoid weights inside chunks of positions, a per-head output gate
 // (weights / softcap / gated: the soft-max variants — pi_attention_weights — with a tanh cap on the scores and no output gate)
+// (mask_kind: `chunk` is the size of position blocks that do not see each other, or of a window that slides with the token; pool > 0: every block of `pool` positions wholly behind the window is seen
+// through the means of its cached keys / values; conv > 0: q, k and v each pass a causal convolution of `conv` taps per channel; qk_norm / pairing / v_norm: pi_op_qkv_prepare_ex's order, pairs and
+// value norm; rot_factor != 1: angle steps stretched by wavelength against rot_original positions (kept below rot_original / rot_high, divided by rot_factor above rot_original / rot_low, blended between))
 struct pi_gate_attention { int heads = 0, kv_heads = 0, dim = 0, vdim = 0, rot_dims = 0, chunk = 0; float rot_base = 10000.0f, scale = 1.0f; int weights = PI_WEIGHTS_SIGMOID; float softcap = 0.0f; bool gated = true;
-                           int in_rows() const { return heads * dim + kv_heads * (dim + vdim) + (gated ? heads : 0); } };         // [q | k | v | gate]
+                           int mask_kind = PI_MASK_CHUNK, pool = 0, conv = 0, qk_norm = PI_QK_NORM_FIRST, pairing = PI_PAIR_HALVES; bool v_norm = true;
+                           float rot_factor = 1.0f, rot_low = 1.0f, rot_high = 1.0f; int rot_original = 0;
+                           int channels() const { return heads * dim + kv_heads * (dim + vdim); }                                  // [q | k | v]
+                           int in_rows() const { return channels() + (gated ? heads : 0); }                                       // [q | k | v | gate]
+                           int cell_rows() const { return pool > 0 && chunk > 0 && mask_kind == PI_MASK_WINDOW ? 2 : 1; }          // cache rows per cell: the token's own, and the pooled block it completes
+                           size_t conv_floats() const { return conv > 1 ? (size_t) (conv - 1) * channels() : 0; } };
 // selective state-space recurrence: a [state][vdim] matrix per head and sequence, B / C shared by the heads of a group, a causal convolution of `conv` taps over x, B, C
 struct pi_ssd { int heads = 0, vdim = 0, state = 0, groups = 0, conv = 0, norm_groups = 1;
                 int inner() const { return heads * vdim; } int channels() const { return inner() + 2 * groups * state; } int in_rows() const { return 2 * inner() + 2 * groups * state + heads; }   // [z | x | B | C | dt]
@@ -73,7 +85,9 @@ struct pi_channel_delta { int heads = 0, kv_heads = 0, dim = 0, vdim = 0, conv =
 struct pi_time_mix { int heads = 0, dim = 0, decay_rank = 0, width = 0;
                      int inner() const { return heads * dim; } size_t matrix_floats() const { return (size_t) heads * dim * dim; } size_t state_floats() const { return matrix_floats() + (size_t) width; } };
 enum pi_mlp_kind { PI_MLP_NONE = 0, PI_MLP_MOE_RELU_SQR = 1 /* routed by a soft-max with correction, experts relu(up)^2, identity experts */, PI_MLP_DENSE_RELU_SQR = 2,
-                   PI_MLP_MOE_GLU = 3 /* routed by sigmoid scores inside the best groups, experts silu(gate) * up, an optional shared expert */, PI_MLP_DENSE_GEGLU = 4 /* down (gelu_tanh(gate) * up) */ };
+                   PI_MLP_MOE_GLU = 3 /* routed by sigmoid scores inside the best groups, experts silu(gate) * up, an optional shared expert */, PI_MLP_DENSE_GEGLU = 4 /* down (gelu_tanh(gate) * up) */,
+                   PI_MLP_DENSE_GELU = 5 /* down gelu(up), the erf form */, PI_MLP_MOE_CLIPPED = 6 /* the `top` largest router logits (+ bias), soft-max over those; experts down(g sigmoid(1.702 g) (u + 1)) with
+                                                                                                       g = min(gate, limit), u = clip(up, +-limit); an optional shared expert of the same form times a per-token sigmoid gate */ };
 struct pi_hybrid_layer {
     pi_mixer_kind mixer = PI_MIXER_LATENT_ATTENTION;
     int weights = 0;                                  // index of the layer that owns the tensors (its own index unless shared)
@@ -84,14 +98,17 @@ struct pi_hybrid_layer {
     pi_channel_delta delta; pi_time_mix shift;                                              // PI_MIXER_CHANNEL_DELTA; PI_MIXER_PARALLEL_SHIFT (beside `left`)
     bool has_mlp = false; int n_expert = 0, n_identity = 0, top = 0, ff = 0;
     pi_mlp_kind mlp = PI_MLP_NONE; int route_groups = 0, route_keep = 0, shared_ff = 0;     // (has_mlp <=> mlp != PI_MLP_NONE)
+    float glu_limit = 0.0f, shared_limit = 0.0f;      // clipped experts: the bound on gate (from above) and up (both sides); 0: none
+    int name_index = -1;                              // the layer of the description whose names the tensors carry (a repeated run lists a layer several times; -1: the entry's own index)
+    bool loop_entry = false;                          // first layer of a repeated run: x <- W_in [x ; embedding row] in front of it
     int cache_index = -1, state_index = -1;           // ordinal among the layers that keep a per-cell cache / a recurrent state
-    int in_rows() const { return mixer == PI_MIXER_CHANNEL_DELTA ? delta.in_rows() : mixer == PI_MIXER_PARALLEL_SHIFT ? left.in_rows() : mixer == PI_MIXER_PARALLEL ? left.in_rows() + right.in_rows() : mixer == PI_MIXER_LIGHTNING ? 2 * heads * dim + 2 * heads * vdim : heads * dim + kv_rank; }     // rows of the fused input projection
-    int out_cols() const { return mixer == PI_MIXER_CHANNEL_DELTA ? delta.heads * delta.vdim : mixer == PI_MIXER_PARALLEL_SHIFT ? std::max(left.heads * left.vdim, shift.inner()) : mixer == PI_MIXER_PARALLEL ? std::max(left.heads * left.vdim, right.inner()) : heads * vdim; }                                                   // widest input of an output projection
-    size_t cell_floats() const { return mixer == PI_MIXER_CHANNEL_DELTA ? 0 : mixer == PI_MIXER_PARALLEL || mixer == PI_MIXER_PARALLEL_SHIFT ? (size_t) left.kv_heads * (left.dim + left.vdim) : mixer == PI_MIXER_LATENT_ATTENTION ? (size_t) kv_rank : 0; }   // cached per cell
-    size_t state_floats() const { return mixer == PI_MIXER_CHANNEL_DELTA ? delta.state_floats() : mixer == PI_MIXER_PARALLEL_SHIFT ? shift.state_floats() : mixer == PI_MIXER_PARALLEL ? right.state_floats() : mixer == PI_MIXER_LIGHTNING ? (size_t) heads * dim * vdim : 0; }                       // kept per sequence
+    int in_rows() const { return mixer == PI_MIXER_CHANNEL_DELTA ? delta.in_rows() : mixer == PI_MIXER_PARALLEL_SHIFT || mixer == PI_MIXER_WINDOW_ATTENTION ? left.in_rows() : mixer == PI_MIXER_PARALLEL ? left.in_rows() + right.in_rows() : mixer == PI_MIXER_LIGHTNING ? 2 * heads * dim + 2 * heads * vdim : heads * dim + kv_rank; }     // rows of the fused input projection
+    int out_cols() const { return mixer == PI_MIXER_CHANNEL_DELTA ? delta.heads * delta.vdim : mixer == PI_MIXER_WINDOW_ATTENTION ? left.heads * left.vdim : mixer == PI_MIXER_PARALLEL_SHIFT ? std::max(left.heads * left.vdim, shift.inner()) : mixer == PI_MIXER_PARALLEL ? std::max(left.heads * left.vdim, right.inner()) : heads * vdim; }                                                   // widest input of an output projection
+    size_t cell_floats() const { return mixer == PI_MIXER_CHANNEL_DELTA ? 0 : mixer == PI_MIXER_WINDOW_ATTENTION ? (size_t) left.cell_rows() * left.kv_heads * (left.dim + left.vdim) : mixer == PI_MIXER_PARALLEL || mixer == PI_MIXER_PARALLEL_SHIFT ? (size_t) left.kv_heads * (left.dim + left.vdim) : mixer == PI_MIXER_LATENT_ATTENTION ? (size_t) kv_rank : 0; }   // cached per cell
+    size_t state_floats() const { return mixer == PI_MIXER_WINDOW_ATTENTION ? (size_t) shift.width + left.conv_floats() : mixer == PI_MIXER_CHANNEL_DELTA ? delta.state_floats() : mixer == PI_MIXER_PARALLEL_SHIFT ? shift.state_floats() : mixer == PI_MIXER_PARALLEL ? right.state_floats() : mixer == PI_MIXER_LIGHTNING ? (size_t) heads * dim * vdim : 0; }                       // kept per sequence
     // a layer's per-sequence state has up to two parts, each stored [slots][part]: the recurrence's matrices, then the convolution's last inputs / the previous token's input
     void state_parts(size_t parts[2]) const {
-        parts[0] = mixer == PI_MIXER_CHANNEL_DELTA ? delta.matrix_floats() : mixer == PI_MIXER_PARALLEL_SHIFT ? shift.matrix_floats() : mixer == PI_MIXER_PARALLEL ? (size_t) right.heads * right.state * right.vdim : state_floats();
+        parts[0] = mixer == PI_MIXER_WINDOW_ATTENTION ? (size_t) shift.width /* the previous token's normed input */ : mixer == PI_MIXER_CHANNEL_DELTA ? delta.matrix_floats() : mixer == PI_MIXER_PARALLEL_SHIFT ? shift.matrix_floats() : mixer == PI_MIXER_PARALLEL ? (size_t) right.heads * right.state * right.vdim : state_floats();
         parts[1] = state_floats() - parts[0];
     }
 };
@@ -107,6 +124,9 @@ struct pi_hybrid_weights {                            // the tensors of a layer 
     // post-norm blocks: layer scales; channel delta: w_in = rows [q | k | v | a1 | g1 | beta], the second halves of the low-rank decay / gate projections; attention + time mix: w_in = [q | k | v], w_o = the
     // attention branch's, the time mix's own projections (each reads its own mix of the input), its shift factors [r | k | v | g | w][width], decay offset, bonus, and both branches' width-norms
     float * ls1 = nullptr, * ls2 = nullptr, * mu = nullptr, * w0 = nullptr, * bonus = nullptr, * left_out = nullptr, * right_out = nullptr;
+    // tanh norms: the scalar inside the tanh (one float on the device); window attention: the learned sink per head (`sink`), the token-shift factors (`mu`); clipped experts: the router's bias (`correction`),
+    // the shared expert [gate | up | its per-token gate row] (ff_up) and down (ff_down); the repeated run's input matrix [width][2 * width] on the entry layer (w_loop)
+    float * norm1_alpha = nullptr; pi_weight * w_loop = nullptr;
     pi_weight * w_a2 = nullptr, * w_g2 = nullptr, * w_r = nullptr, * w_k = nullptr, * w_v = nullptr, * w_g = nullptr, * w_w1 = nullptr, * w_w2 = nullptr, * w_o2 = nullptr;
     bool loaded = false;
 };
@@ -125,7 +145,9 @@ struct pi_hparams {
     // ... or the norm after the sum: x <- R(post_alpha * x + ls * sublayer(x)) * w.  pair_buckets > 0: the embedding adds row (previous token * pair_mul_prev + token * pair_mul_cur) mod pair_buckets
     // of a second table (row pair_buckets for a sequence's first token); the previous token is part of a sequence's state (state_slots)
     bool post_norm = false; float post_alpha = 1.0f; int pair_buckets = 0, pair_mul_prev = 0, pair_mul_cur = 0;
-    bool hybrid_arch() const { return arch == PI_ARCH_FASOVIK || arch == PI_ARCH_VIKARAX || arch == PI_ARCH_RAFUSUN; }
+    // ... or ONE norm per layer, tanh(alpha x) * w + b, whose output the mixer (token-shifted) and the feed-forward both read: x <- x + mixer(shift(h)) + ff(h)
+    bool shared_tanh_norm = false;
+    bool hybrid_arch() const { return arch == PI_ARCH_FASOVIK || arch == PI_ARCH_VIKARAX || arch == PI_ARCH_RAFUSUN || arch == PI_ARCH_RAREVIK; }
     int n_latent() const { int n = 0; for (const auto & l : hybrid) n += l.cache_index >= 0; return n; }
     int n_recurrent() const { int n = 0; for (const auto & l : hybrid) n += l.state_index >= 0; return n; }
     int head_dim() const { return n_embd / n_head; }
@@ -154,6 +176,7 @@ struct llama_model {
     uint64_t n_elements = 0, n_bytes = 0;
     pi_weight * pair_embd = nullptr;                                                               // hashed pair embedding [pair_buckets + 1][n_embd]
     pi_weight * tok_embd = nullptr, * output = nullptr, * pos_embd = nullptr;                 // pos_embd: StarCoder's learned positions (llama.cpp:4251-4255)
+    float * output_norm_alpha = nullptr;                                                         // tanh norms: the final norm's scalar (one float on the device)
     float * output_norm = nullptr, * output_norm_b = nullptr, * tok_norm = nullptr, * tok_norm_b = nullptr;   // tok_norm: Bloom's LayerNorm on the embeddings (llama.cpp:4650-4654)
     float * alibi_slopes = nullptr;                                                              // f32 [n_head] on the device when block.alibi > 0
     std::vector<pi_layer> layers;
@@ -242,6 +265,7 @@ struct llama_context {
     // a mixer's two branches do not depend on each other between the in- and the out-projection: with PI_BRANCH_STREAMS=1 the second one runs on a stream of its own (forked and joined
     // by events, inside the captured graph as well as in eager launches) so that its small dependent kernels overlap the first one's
     hipStream_t branch_stream = nullptr; std::vector<hipEvent_t> branch_events;     // [2 * layer]: fork, join
+    float * x_pair = nullptr, * h_out3 = nullptr;             // repeated runs: rows [x | embedding row] that the run's input matrix reads; a third sublayer output (the shared expert's)
     float * hist = nullptr, * h_out2 = nullptr, * ssd_dt = nullptr;   // depth average: the stream after the embedding and after every layer [n_layer + 1][n_batch][width]; second branch output; step sizes | decays
     std::unique_ptr<pi::state_slots> slots; int n_state_slots = 8;
     int32_t * rec_dev = nullptr;                              // per token of the pass: state slot (| 1 << 30: start from zero)

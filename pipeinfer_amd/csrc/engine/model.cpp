@@ -196,6 +196,12 @@ size_t llama_model::stage_weight_bytes(int l0, int l1, bool first, bool last, in
                 b += 4 * 4 * w + (H.has_mlp ? 6 * (size_t) H.ff * w : 0);
                 continue;
             }
+            if (H.mixer == PI_MIXER_WINDOW_ATTENTION) {                        // the projections, the norm's and the shift's vectors, the convolution taps, the feed-forward a token uses, a repeated run's input matrix
+                b += 2 * ((size_t) H.in_rows() + (size_t) H.left.heads * H.left.vdim) * w + 4 * 4 * w + 4 * (size_t) H.left.channels() * H.left.conv + (H.loop_entry ? 4 * w * w : 0);
+                if (H.mlp == PI_MLP_DENSE_GELU) b += 4 * (size_t) H.ff * w;
+                if (H.mlp == PI_MLP_MOE_CLIPPED) b += 2 * (size_t) H.n_expert * w + (size_t) std::min(H.n_expert, std::max(1, n_tok) * H.top) * 6 * (size_t) H.ff * w + (H.shared_ff > 0 ? 6 * (size_t) H.shared_ff * w + 2 * w : 0);
+                continue;
+            }
             if (H.mixer == PI_MIXER_PARALLEL) {                                // both branches' projections, the norms' vectors, the feed-forward a token uses
                 b += 2 * (size_t) H.in_rows() * w + 2 * ((size_t) H.left.heads * H.left.vdim + H.right.inner()) * w + 4 * 8 * w;
                 if (H.mlp == PI_MLP_DENSE_RELU_SQR) b += 4 * (size_t) H.ff * w;
@@ -314,7 +320,7 @@ extern "C" enum llama_vocab_type llama_vocab_type(const struct llama_model * m) 
 extern "C" uint64_t llama_model_size(const struct llama_model * m) { return m->n_bytes; }
 extern "C" uint64_t llama_model_n_params(const struct llama_model * m) { return m->n_elements; }
 extern "C" int llama_model_desc(const struct llama_model * m, char * buf, size_t n) {
-    static const char * names[] = { "llama", "falcon", "baichuan", "starcoder", "refact", "bloom", "mpt", "stablelm", "persimmon", "fasovik", "vikarax", "rafusun" };
+    static const char * names[] = { "llama", "falcon", "baichuan", "starcoder", "refact", "bloom", "mpt", "stablelm", "persimmon", "fasovik", "vikarax", "rafusun", "rarevik" };
     return snprintf(buf, n, "%s %s", names[m->hparams.arch], m->name.c_str());
 }
 

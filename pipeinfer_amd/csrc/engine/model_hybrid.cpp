@@ -14,6 +14,12 @@
 // or { type: "parallel", mixer: { left: { heads, kv_heads, dim, vdim, scale, softcap, rot.dims / rot.base, mask.size }, right: { heads, dim } } }, mlp: null | { kind: "dense", ff }.  The ranks of the low-rank
 // projections are the tensors' own.  Tensors: embed, bigram, head, final.norm, l<i>.norm1 / norm2, l<i>.ls1 / ls2, l<i>.mix.{q, k, v (+ .conv), b, A_log, dt_bias, a1, a2, g1, g2, norm, o} or
 // l<i>.mix.left.{q, k, v, o, out}, l<i>.mix.right.{mu.{r, k, v, g, w}, r, k, v, g, w1, w2, w0, u, norm, o, out}, l<i>.mlp.{gate, up, down}.
+//
+// Rarevik (same files, other keys): vocab, width, norm.eps, loop.{start, stop, times} (optional: layers [start, stop) run `times` times in a row with the same tensors, each run with a cache and state of
+// its own), layers[]: { type: "attention", mixer: { heads, kv_heads, dim, vdim, scale, conv, rot.dims / rot.base, mask.size / mask.pool } } or { type: "attention_2", mixer: { heads, kv_heads, dim, vdim,
+// scale, rot.dims / rot.base / rot.scaling.{factor, low, high, original}, mask.size } }, mlp: null | { kind: "dense", ff } | { kind: "moe", expert.ff / expert.limit, router.experts / router.top,
+// shared.ff / shared.limit }.  Tensors: embed, loop.in, final.norm (+ .b, .alpha), l<i>.norm1 (+ .b, .alpha), l<i>.shift, l<i>.mix.{q, k, v, o} with {q.conv, k.conv, v.conv, q.norm, k.norm, sink} or {g},
+// l<i>.mlp.{up, down} or l<i>.mlp.{router, router.b, e<k>.{gate, up, down}, shared.{gate, up, down, sg}}.
 #include "engine.h"
 #include "json.h"
 
@@ -104,6 +110,11 @@ struct loader {
             for (size_t i = 0; i < n; i++) v[at + i] = bf16_to_f32(((const uint16_t *) t->data)[i]);
         }
         return vector_f32(v);
+    }
+    float * scalar(const std::string & name) {                                  // a tensor without dimensions: one float on the device
+        const pi::st_tensor * t = get(name, {});
+        if (!t) return nullptr;
+        return vector_f32({ bf16_to_f32(((const uint16_t *) t->data)[0]) });
     }
     float * vector(const std::string & name, int64_t n) {
         const pi::st_tensor * t = get(name, { n });
@@ -245,6 +256,94 @@ static bool read_rafusun_config(const pi::json & cfg, const pi::safetensors_file
     return true;
 }
 
+// Rarevik: every layer has ONE tanh norm that its mixer (through a token shift) and its feed-forward read; the mixers are sliding-window attentions of two kinds; a run of layers may repeat
+static bool read_rarevik_config(const pi::json & cfg, pi_hparams & hp, std::string & what) {
+    using pi::json;
+    double d;
+    if (!num_at(cfg, "norm.eps", d)) { what = "no 'norm.eps'"; return false; }
+    hp.f_norm_eps = hp.f_norm_rms_eps = (float) d;
+    hp.shared_tanh_norm = true;
+    const json * layers = cfg.find("layers");
+    if (!layers || !layers->is_arr() || layers->arr.empty()) { what = "'layers' must be a non-empty list"; return false; }
+    const int n_desc = (int) layers->arr.size();
+    std::vector<pi_hybrid_layer> desc;
+    for (int i = 0; i < n_desc; i++) {
+        const json & jl = layers->arr[(size_t) i];
+        const std::string where = "layers[" + std::to_string(i) + "]: ";
+        auto bad = [&](const std::string & w) { what = where + w; return false; };
+        pi_hybrid_layer H;
+        H.mixer = PI_MIXER_WINDOW_ATTENTION; H.name_index = i;
+        pi_gate_attention & A = H.left;
+        const json * type = jl.find("type");
+        if (!type || !type->is_str()) return bad("no 'type'");
+        const bool pooled_kind = type->str == "attention";
+        if (!pooled_kind && type->str != "attention_2") return bad("mixer type '" + type->str + "' is unknown (attention, attention_2)");
+        if (!int_at(jl, "mixer.heads", A.heads) || !int_at(jl, "mixer.kv_heads", A.kv_heads) || !int_at(jl, "mixer.dim", A.dim) || !int_at(jl, "mixer.vdim", A.vdim) ||
+            A.heads < 1 || A.kv_heads < 1 || A.heads % A.kv_heads || A.dim < 1 || A.vdim < 1) return bad("mixer needs positive 'heads', 'kv_heads' (a divisor of heads), 'dim', 'vdim'");
+        if (!num_at(jl, "mixer.scale", d)) return bad("mixer needs 'scale'");
+        A.scale = (float) d; A.weights = PI_WEIGHTS_SOFTMAX; A.v_norm = false; A.mask_kind = PI_MASK_WINDOW;
+        if (jl.at("mixer.rot") && !jl.at("mixer.rot")->is_null()) {
+            if (!int_at(jl, "mixer.rot.dims", A.rot_dims) || !num_at(jl, "mixer.rot.base", d) || (A.rot_dims & 1) || A.rot_dims > A.dim || d <= 0) return bad("mixer.rot needs an even 'dims' <= dim and a positive 'base'");
+            A.rot_base = (float) d;
+        }
+        if (jl.at("mixer.mask") && !jl.at("mixer.mask")->is_null() && (!int_at(jl, "mixer.mask.size", A.chunk) || A.chunk < 1)) return bad("mixer.mask needs a positive 'size'");
+        if (pooled_kind) {                                                  // a short convolution behind the projections, normed q / k turned in halves, pooled far blocks, a learned sink
+            A.gated = false; A.qk_norm = PI_QK_NORM_FIRST; A.pairing = PI_PAIR_HALVES;
+            if (jl.at("mixer.conv") && !jl.at("mixer.conv")->is_null() && (!int_at(jl, "mixer.conv", A.conv) || A.conv < 1 || A.conv > 64)) return bad("mixer.conv must lie between 1 and 64");
+            if (A.chunk > 0 && jl.at("mixer.mask.pool") && !jl.at("mixer.mask.pool")->is_null() && (!int_at(jl, "mixer.mask.pool", A.pool) || A.pool < 1 || A.pool > 8192)) return bad("mixer.mask.pool must lie between 1 and 8192");
+        } else {                                                            // q / k turned in neighbouring pairs by (possibly stretched) angle steps, no norms, a sigmoid gate per head
+            A.gated = true; A.qk_norm = PI_QK_NORM_NONE; A.pairing = PI_PAIR_NEIGHBOURS;
+            if (A.rot_dims > 0 && jl.at("mixer.rot.scaling") && !jl.at("mixer.rot.scaling")->is_null()) {
+                double f, lo, hi;
+                if (!num_at(jl, "mixer.rot.scaling.factor", f) || !num_at(jl, "mixer.rot.scaling.low", lo) || !num_at(jl, "mixer.rot.scaling.high", hi) || !int_at(jl, "mixer.rot.scaling.original", A.rot_original) ||
+                    f <= 0 || lo <= 0 || hi <= 0 || A.rot_original < 1) return bad("mixer.rot.scaling needs positive 'factor', 'low', 'high' and 'original'");
+                A.rot_factor = (float) f; A.rot_low = (float) lo; A.rot_high = (float) hi;
+            }
+        }
+        H.heads = A.heads; H.dim = A.dim; H.vdim = A.vdim; H.shift.width = hp.n_embd;
+        if (jl.has("mlp")) {
+            const json * kind = jl.at("mlp.kind");
+            if (!kind || !kind->is_str()) return bad("mlp needs 'kind'");
+            if (kind->str == "dense") {
+                if (!int_at(jl, "mlp.ff", H.ff) || H.ff < 1) return bad("a dense mlp needs 'ff'");
+                H.mlp = PI_MLP_DENSE_GELU;
+            } else if (kind->str == "moe") {
+                if (!int_at(jl, "mlp.router.experts", H.n_expert) || !int_at(jl, "mlp.router.top", H.top) || !int_at(jl, "mlp.expert.ff", H.ff) || H.n_expert < 1 || H.ff < 1 || H.top < 1 || H.top > H.n_expert)
+                    return bad("a routed mlp needs 'router.experts', 'router.top' (at most the experts), 'expert.ff'");
+                if (num_at(jl, "mlp.expert.limit", d)) { if (d <= 0) return bad("mlp.expert.limit must be positive"); H.glu_limit = (float) d; }
+                if (jl.at("mlp.shared") && !jl.at("mlp.shared")->is_null()) {
+                    if (!int_at(jl, "mlp.shared.ff", H.shared_ff) || H.shared_ff < 1) return bad("mlp.shared needs 'ff'");
+                    if (num_at(jl, "mlp.shared.limit", d)) { if (d <= 0) return bad("mlp.shared.limit must be positive"); H.shared_limit = (float) d; }
+                }
+                H.mlp = PI_MLP_MOE_CLIPPED;
+            } else return bad("feed-forward kind '" + kind->str + "' is unknown (dense, moe)");
+            H.has_mlp = true;
+        }
+        desc.push_back(std::move(H));
+    }
+    // the order the layers run in: [0, start) once, [start, stop) `times` times, [stop, n) once.  Every entry of the run list is a layer of its own to the context (cache, state); its tensors are those of
+    // the first run of the same description
+    int start = n_desc, stop = n_desc, times = 1;
+    if (cfg.at("loop") && !cfg.at("loop")->is_null()) {
+        if (!int_at(cfg, "loop.start", start) || !int_at(cfg, "loop.stop", stop) || !int_at(cfg, "loop.times", times) || start > stop || stop > n_desc || times > 4096) { what = "'loop' needs 0 <= start <= stop <= layers and 'times'"; return false; }
+    }
+    std::vector<int> first_run((size_t) n_desc, -1);
+    auto add = [&](int i, bool entry) {
+        pi_hybrid_layer H = desc[(size_t) i];
+        const int r = (int) hp.hybrid.size();
+        if (first_run[(size_t) i] < 0) first_run[(size_t) i] = r;
+        H.weights = first_run[(size_t) i]; H.loop_entry = entry; H.cache_index = r; H.state_index = r;
+        hp.hybrid.push_back(std::move(H));
+    };
+    for (int i = 0; i < start; i++) add(i, false);
+    for (int k = 0; k < times; k++) for (int i = start; i < stop; i++) add(i, i == start);
+    for (int i = stop; i < n_desc; i++) add(i, false);
+    if (hp.hybrid.empty()) { what = "no layer runs"; return false; }
+    hp.n_layer = (int) hp.hybrid.size();
+    hp.n_head = hp.n_head_kv = 1; hp.n_ctx_train = 0;
+    return true;
+}
+
 }  // namespace
 
 bool llama_model::ensure_loaded_hybrid(int n_positions, std::string & err) {
@@ -261,17 +360,49 @@ bool llama_model::ensure_loaded_hybrid(int n_positions, std::string & err) {
         if (!(output = L.matrix({ { "head", hp.n_vocab } }, width))) return false;
         if (!hp.post_norm && !(output_norm_b = L.vector("final.norm.b", width))) return false;
     }
+    if (hp.shared_tanh_norm && !output_norm_alpha && (!(output_norm_b = L.vector("final.norm.b", width)) || !(output_norm_alpha = L.scalar("final.norm.alpha")))) return false;
     if (hp.pair_buckets > 0 && !pair_embd && !(pair_embd = L.matrix({ { "bigram", (int64_t) hp.pair_buckets + 1 } }, width))) return false;
     for (size_t i = 0; i < hp.hybrid.size(); i++) {
         const pi_hybrid_layer & H = hp.hybrid[i];
         pi_hybrid_weights & W = hweights[i];
         if (H.weights == (int) i && W.loaded && W.rotary && pi_rotary_table_positions(W.rotary) < n_positions) {        // a later context is longer than the table
-            void * t = pi_rotary_table_create(n_positions, H.left.rot_dims, H.left.rot_base);
+            void * t = pi_rotary_table_create_scaled(n_positions, H.left.rot_dims, H.left.rot_base, H.left.rot_factor, H.left.rot_low, H.left.rot_high, H.left.rot_original);
             if (!t) { err = std::string("rotation table: ") + pi_last_error(); return false; }
             retired_tables.push_back(W.rotary); W.rotary = t;
         }
         if (H.weights != (int) i || W.loaded) continue;
-        const std::string p = "l" + std::to_string(i) + ".";
+        const std::string p = "l" + std::to_string(H.name_index >= 0 ? H.name_index : (int) i) + ".";
+        if (hp.shared_tanh_norm) {                                         // one tanh norm per layer; window attention; dense or routed clipped feed-forward
+            if (H.mixer != PI_MIXER_WINDOW_ATTENTION) { err = "a block with one shared tanh norm has no mixer of kind " + std::to_string((int) H.mixer); return false; }
+            const pi_gate_attention & A = H.left;
+            const std::string m = p + "mix.";
+            const int64_t hd = (int64_t) A.heads * A.dim, gd = (int64_t) A.kv_heads * A.dim, gv = (int64_t) A.kv_heads * A.vdim;
+            if (!(W.norm1 = L.vector(p + "norm1", width)) || !(W.norm1_b = L.vector(p + "norm1.b", width)) || !(W.norm1_alpha = L.scalar(p + "norm1.alpha")) || !(W.mu = L.vector(p + "shift", width))) return false;
+            std::vector<std::pair<std::string, int64_t>> in_parts = { { m + "q", hd }, { m + "k", gd }, { m + "v", gv } };
+            if (A.gated) in_parts.push_back({ m + "g", A.heads });
+            if (!(W.w_in = L.matrix(in_parts, width)) || !(W.w_o = L.matrix({ { m + "o", width } }, (int64_t) A.heads * A.vdim))) return false;
+            if (A.conv > 0 && !(W.conv_w = L.vectors({ { m + "q.conv", hd }, { m + "k.conv", gd }, { m + "v.conv", gv } }, A.conv))) return false;
+            if (A.qk_norm != PI_QK_NORM_NONE && (!(W.q_norm = L.vector(m + "q.norm", A.dim)) || !(W.k_norm = L.vector(m + "k.norm", A.dim)))) return false;
+            if (!A.gated && !(W.sink = L.vector(m + "sink", A.heads))) return false;
+            if (!(W.rotary = pi_rotary_table_create_scaled(std::max(n_positions, 32), A.rot_dims, A.rot_base, A.rot_factor, A.rot_low, A.rot_high, A.rot_original))) { err = std::string("rotation table: ") + pi_last_error(); return false; }
+            if (H.mlp == PI_MLP_DENSE_GELU) {
+                if (!(W.ff_up = L.matrix({ { p + "mlp.up", H.ff } }, width)) || !(W.ff_down = L.matrix({ { p + "mlp.down", width } }, H.ff))) return false;
+            } else if (H.mlp == PI_MLP_MOE_CLIPPED) {
+                if (!(W.router = L.matrix({ { p + "mlp.router", H.n_expert } }, width)) || !(W.correction = L.vector(p + "mlp.router.b", H.n_expert))) return false;
+                std::vector<std::pair<std::string, int64_t>> ups, downs;
+                for (int e = 0; e < H.n_expert; e++) {
+                    const std::string q = p + "mlp.e" + std::to_string(e) + ".";
+                    ups.push_back({ q + "gate", H.ff }); ups.push_back({ q + "up", H.ff }); downs.push_back({ q + "down", width });
+                }
+                if (!(W.e_up = L.matrix(ups, width)) || !(W.e_down = L.matrix(downs, H.ff))) return false;
+                // the shared expert's per-token gate is one more row of its first matrix: [gate | up | sg]
+                if (H.shared_ff > 0 && (!(W.ff_up = L.matrix({ { p + "mlp.shared.gate", H.shared_ff }, { p + "mlp.shared.up", H.shared_ff }, { p + "mlp.shared.sg", 1 } }, width)) ||
+                                        !(W.ff_down = L.matrix({ { p + "mlp.shared.down", width } }, H.shared_ff)))) return false;
+            }
+            if (H.loop_entry && !(W.w_loop = L.matrix({ { "loop.in", width } }, 2 * width))) return false;
+            W.loaded = true;
+            continue;
+        }
         if (hp.post_norm) {                                                // the norm after the sum: per sublayer a norm and a layer scale
             if (!(W.norm1 = L.vector(p + "norm1", width)) || !(W.ls1 = L.vector(p + "ls1", width))) return false;
             if (H.has_mlp && (!(W.norm2 = L.vector(p + "norm2", width)) || !(W.ls2 = L.vector(p + "ls2", width)))) return false;
@@ -388,19 +519,20 @@ llama_model * load_hybrid_model(const std::string & folder, const llama_model_pa
     if (arch->str == "Fasovik") hp.arch = PI_ARCH_FASOVIK;
     else if (arch->str == "Vikarax") hp.arch = PI_ARCH_VIKARAX;
     else if (arch->str == "Rafusun") hp.arch = PI_ARCH_RAFUSUN;
-    else return fail("architecture '" + arch->str + "' is not one this engine builds (Fasovik, Vikarax, Rafusun)");
+    else if (arch->str == "Rarevik") hp.arch = PI_ARCH_RAREVIK;
+    else return fail("architecture '" + arch->str + "' is not one this engine builds (Fasovik, Vikarax, Rafusun, Rarevik)");
     m->name = arch->str;
     double d;
     if (!int_at(cfg, "vocab", hp.n_vocab) || !int_at(cfg, "width", hp.n_embd) || hp.n_vocab < 1 || hp.n_embd < 1) return fail("'vocab' and 'width' must be positive integers");
-    if (hp.arch == PI_ARCH_VIKARAX || hp.arch == PI_ARCH_RAFUSUN) {
+    if (hp.arch == PI_ARCH_VIKARAX || hp.arch == PI_ARCH_RAFUSUN || hp.arch == PI_ARCH_RAREVIK) {
         std::string what;
         if (!params.vocab_only && !m->st_file.open(folder + "/model.safetensors", err)) { fprintf(stderr, "llama_load_model_from_file: %s\n", err.c_str()); return nullptr; }
-        if (hp.arch == PI_ARCH_VIKARAX ? !read_vikarax_config(cfg, hp, what) : !read_rafusun_config(cfg, params.vocab_only ? nullptr : &m->st_file, hp, what)) return fail(what);
+        if (hp.arch == PI_ARCH_VIKARAX ? !read_vikarax_config(cfg, hp, what) : hp.arch == PI_ARCH_RAREVIK ? !read_rarevik_config(cfg, hp, what) : !read_rafusun_config(cfg, params.vocab_only ? nullptr : &m->st_file, hp, what)) return fail(what);
         m->hweights.resize((size_t) hp.n_layer);
         if (!params.vocab_only) {
             for (const auto & kv : m->st_file.tensors) { m->n_elements += (uint64_t) kv.second.elements(); m->n_bytes += kv.second.nbytes; }
             const st_tensor * e = m->st_file.tensor("embed"), * h = m->st_file.tensor("head");
-            if (!e || e->shape != std::vector<int64_t>{ hp.n_vocab, hp.n_embd } || !h || h->shape != e->shape) return fail("tensors 'embed' and 'head' are missing or not [vocab][width]");
+            if (!e || e->shape != std::vector<int64_t>{ hp.n_vocab, hp.n_embd } || (hp.arch != PI_ARCH_RAREVIK && (!h || h->shape != e->shape))) return fail("tensors 'embed' and 'head' are missing or not [vocab][width]");
         }
         return m.release();
     }

@@ -32,6 +32,7 @@ static __device__ __forceinline__ float dn_act(float v, int act) {
         case PI_ACT_RELU_SQR: { const float r = fmaxf(v, 0.0f); return r * r; }
         case PI_ACT_TANH:     return tanhf(v);
         case PI_ACT_GELU_TANH: return 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));
+        case PI_ACT_GELU_ERF: return 0.5f * v * (1.0f + erff(v * 0.7071067811865476f));
         default:              return v;
     }
 }

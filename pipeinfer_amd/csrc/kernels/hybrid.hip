@@ -342,6 +342,66 @@ extern "C" int pi_op_glu_mul(const float * in, int64_t in_stride, int ff, int n_
     PI_CHECK_LAUNCH(); return 0;
 }
 
+// a gated hidden layer from its raw halves: PI_GLU_SILU silu(g) * u; PI_GLU_CLIPPED g' sigmoid(1.702 g') (u' + 1) with g' = min(g, limit), u' = clip(u, -limit, limit) (limit <= 0: no bounds)
+static __device__ __forceinline__ float hy_glu(float g, float u, int glu, float limit) {
+    if (glu == PI_GLU_CLIPPED) {
+        if (limit > 0.0f) { g = fminf(g, limit); u = fminf(fmaxf(u, -limit), limit); }
+        return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+    }
+    return glu == PI_GLU_SILU ? g / (1.0f + expf(-g)) * u : g * u;
+}
+__global__ void k_glu_mul_ex(const float * __restrict__ in, int64_t is, int ff, int glu, float limit, int64_t gate_col, float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.y, f = blockIdx.x * 256 + threadIdx.x;
+    if (f >= ff) return;
+    const float * r = in + (int64_t) t * is;
+    float y = hy_glu(r[f], r[ff + f], glu, limit);
+    if (gate_col >= 0) y *= 1.0f / (1.0f + expf(-r[gate_col]));
+    out[(int64_t) t * os + f] = y;
+}
+extern "C" int pi_op_glu_mul_ex(const float * in, int64_t in_stride, int ff, int glu, float limit, int64_t gate_col, int n_tok, float * out, int64_t out_stride, void * stream) {
+    if (n_tok <= 0 || ff <= 0) return 0;
+    if (glu < PI_GLU_OFF || glu > PI_GLU_CLIPPED || gate_col >= in_stride) { pi_set_error("pi_op_glu_mul_ex: hidden layer of kind %d, gate column %lld of rows %lld floats apart", glu, (long long) gate_col, (long long) in_stride); return -1; }
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 12.0 * ff * n_tok, k_glu_mul_ex, dim3((unsigned) ((ff + 255) / 256), (unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, in, in_stride, ff, glu, limit, gate_col, out, out_stride, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+
+// ---- rows of the stream: copies, and a layer's end with the next tanh norm --------------------------------------------------------------------------------------
+__global__ void k_copy_rows(const float * __restrict__ src, int64_t ss, float * __restrict__ dst, int64_t ds, int n, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.y, i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[(int64_t) t * ds + i] = src[(int64_t) t * ss + i];
+}
+extern "C" int pi_op_copy_rows(const float * src, int64_t src_stride, float * dst, int64_t dst_stride, int n, int n_tok, void * stream) {
+    if (n_tok <= 0 || n <= 0) return 0;
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 8.0 * n * n_tok, k_copy_rows, dim3((unsigned) ((n + 255) / 256), (unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, src, src_stride, dst, dst_stride, n, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+// x_out = x + a + b + c (summed in this order); h = tanh(alpha * x_out) * w + bias: no statistics, so a thread needs nobody else's values
+__global__ void k_sum_tanh_norm(const float * __restrict__ x, int64_t xs, const float * __restrict__ a, int64_t as, const float * __restrict__ b, int64_t bs, const float * __restrict__ c, int64_t cs, int n,
+                                float * __restrict__ xo, int64_t xos, const float * __restrict__ alpha, const float * __restrict__ w, const float * __restrict__ bias, float * __restrict__ ho, int64_t hos,
+                                const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.y, i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float v = x[(int64_t) t * xs + i];
+    if (a) v += a[(int64_t) t * as + i];
+    if (b) v += b[(int64_t) t * bs + i];
+    if (c) v += c[(int64_t) t * cs + i];
+    if (xo) xo[(int64_t) t * xos + i] = v;
+    if (w) ho[(int64_t) t * hos + i] = fmaf(tanhf(alpha[0] * v), w[i], bias ? bias[i] : 0.0f);
+}
+extern "C" int pi_op_sum_tanh_norm(const float * x, int64_t x_stride, const float * a, int64_t a_stride, const float * b, int64_t b_stride, const float * c, int64_t c_stride, int n, int n_tok,
+                                   float * x_out, int64_t x_out_stride, const float * alpha_dev, const float * w_dev, const float * bias_dev, float * h_out, int64_t h_out_stride, void * stream) {
+    if (n_tok <= 0 || n <= 0) return 0;
+    if (w_dev && (!alpha_dev || !h_out)) { pi_set_error("pi_op_sum_tanh_norm: the norm needs its scalar and an output"); return -1; }
+    if (!w_dev && !x_out) return 0;
+    const int rows = 1 + (a != nullptr) + (b != nullptr) + (c != nullptr) + (x_out != nullptr) + (w_dev != nullptr);
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 4.0 * n * n_tok * rows, k_sum_tanh_norm, dim3((unsigned) ((n + 255) / 256), (unsigned) n_tok), dim3(256), 0, (hipStream_t) stream, x, x_stride, a, a_stride, b, b_stride, c, c_stride, n,
+                 x_out, x_out_stride, alpha_dev, w_dev, bias_dev, h_out, h_out_stride, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+
 // ---- linear attention with a per-head decay -------------------------------------------------------------------------------------------------------
 // rec[t] = state slot of token t (| 1 << 30 on the first token of a sequence whose state starts from zero), tokens of one slot are consecutive.  Workgroup (head, column block,
 // piece): thread (column j, part sp of R) keeps S[i][j] for its DPT rows i in registers and walks the piece's tokens in order.
@@ -931,7 +991,9 @@ __global__ void __launch_bounds__(256) k_moe_route(const uint16_t * __restrict__
     }
     __syncthreads();
     if (wave != 0) return;
-    if (n_groups > 0) {
+    if (n_groups < 0) {                           // by logit (+ bias); the weights are worked out over the chosen ones below
+        for (int e = lane; e < n_out; e += 64) { z[e] += corr ? corr[e] : 0.0f; ch[e] = z[e]; }
+    } else if (n_groups > 0) {
         const int per = n_out / n_groups;
         for (int e = lane; e < n_out; e += 64) { z[e] = 1.0f / (1.0f + expf(-z[e])); ch[e] = -INFINITY; }
         for (int g = lane; g < n_groups; g += 64) {
@@ -969,12 +1031,19 @@ __global__ void __launch_bounds__(256) k_moe_route(const uint16_t * __restrict__
         if (bi == 0x7fffffff) bi = 0;             // (fewer finite choices than `top`: cannot happen with finite logits)
         if (lane == 0) { sel[(int64_t) t * top + kk] = bi; selw[(int64_t) t * top + kk] = z[bi]; ch[bi] = -INFINITY; }
     }
+    if (n_groups < 0 && lane == 0) {              // soft-max over the chosen logits alone (the first chosen is the largest)
+        float * wt = selw + (int64_t) t * top;
+        const float m = wt[0];
+        float l = 0.0f;
+        for (int kk = 0; kk < top; kk++) { wt[kk] = expf(wt[kk] - m); l += wt[kk]; }
+        for (int kk = 0; kk < top; kk++) wt[kk] = wt[kk] / l;
+    }
 }
 
 // up[t][kk][f] = relu(W_up[e] x_t)^2 for the kk-th chosen expert e of token t (nothing for identity experts); a wave per row f.
 // glu: an expert's first matrix holds 2 * ff rows [gate | up] and up[t][kk][f] = silu(gate_f . x) * (up_f . x)
 __global__ void __launch_bounds__(256) k_moe_up(const uint16_t * __restrict__ wup, int64_t width, int ff, int n_exp, const float * __restrict__ x, int64_t xs, const int32_t * __restrict__ sel,
-                                                int top, int exact, int vec, int glu, float * __restrict__ up, const int32_t * __restrict__ abort_w) {
+                                                int top, int exact, int vec, int glu, float limit, float * __restrict__ up, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 0)) return;
     const int lane = threadIdx.x & 63, f = blockIdx.x * 4 + (threadIdx.x >> 6);
     const int slot = blockIdx.y, e = sel[slot];
@@ -984,7 +1053,7 @@ __global__ void __launch_bounds__(256) k_moe_up(const uint16_t * __restrict__ wu
     if (glu) {
         const float g = pi_lanes_sum<64>(hy_dot_lane(wup + ((int64_t) e * 2 * ff + f) * width, xr, width, lane, exact != 0, vec != 0));
         const float u = pi_lanes_sum<64>(hy_dot_lane(wup + ((int64_t) e * 2 * ff + ff + f) * width, xr, width, lane, exact != 0, vec != 0));
-        if (lane == 0) up[(int64_t) slot * ff + f] = g / (1.0f + expf(-g)) * u;
+        if (lane == 0) up[(int64_t) slot * ff + f] = hy_glu(g, u, glu, limit);
         return;
     }
     const float a = pi_lanes_sum<64>(hy_dot_lane(wup + ((int64_t) e * ff + f) * width, xr, width, lane, exact != 0, vec != 0));
@@ -1021,6 +1090,9 @@ static int moe_route_launch(const pi_weight * router, const float * correction_d
 extern "C" int pi_op_moe_route(const pi_weight * router, const float * correction_dev, const float * x, int64_t x_stride, int n_tok, int top, int exact, int32_t * sel_dev, float * selw_dev, void * stream) {
     return moe_route_launch(router, correction_dev, x, x_stride, n_tok, top, exact, 0, 0, sel_dev, selw_dev, stream);
 }
+extern "C" int pi_op_moe_route_top_logits(const pi_weight * router, const float * bias_dev, const float * x, int64_t x_stride, int n_tok, int top, int exact, int32_t * sel_dev, float * selw_dev, void * stream) {
+    return moe_route_launch(router, bias_dev, x, x_stride, n_tok, top, exact, -1, 0, sel_dev, selw_dev, stream);
+}
 extern "C" int pi_op_moe_route_groups(const pi_weight * router, const float * x, int64_t x_stride, int n_tok, int top, int n_groups, int keep, int exact, int32_t * sel_dev, float * selw_dev, void * stream) {
     if (!router || n_groups < 1 || router->ne1 % n_groups || keep < 1 || keep > n_groups || (int64_t) keep * (router->ne1 / n_groups) < top) {
         pi_set_error("pi_op_moe_route_groups: the router's outputs must divide into the groups, and the kept groups must hold at least `top` outputs"); return -1;
@@ -1034,7 +1106,12 @@ extern "C" int pi_op_moe_experts(const pi_weight * wup, const pi_weight * wdown,
 }
 extern "C" int pi_op_moe_experts_act(const pi_weight * wup, const pi_weight * wdown, int n_exp, int ff, int glu, const float * x, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,
                                      int exact, float * up_dev, float * out, int64_t out_stride, void * stream) {
+    return pi_op_moe_experts_glu(wup, wdown, n_exp, ff, glu, 0.0f, x, x_stride, sel_dev, selw_dev, n_tok, top, exact, up_dev, out, out_stride, stream);
+}
+extern "C" int pi_op_moe_experts_glu(const pi_weight * wup, const pi_weight * wdown, int n_exp, int ff, int glu, float limit, const float * x, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok,
+                                     int top, int exact, float * up_dev, float * out, int64_t out_stride, void * stream) {
     if (n_tok <= 0) return 0;
+    if (glu < PI_GLU_OFF || glu > PI_GLU_CLIPPED) { pi_set_error("pi_op_moe_experts: hidden layer of kind %d is unknown", glu); return -1; }
     const int upr = glu ? 2 : 1;                                       // rows of an expert's first matrix, in units of ff
     hipStream_t s = (hipStream_t) stream;
     int64_t width = 0;
@@ -1046,7 +1123,7 @@ extern "C" int pi_op_moe_experts_act(const pi_weight * wup, const pi_weight * wd
         const double b_up = std::min<double>(n_tok * top, n_exp) * 2.0 * upr * ff * width + 4.0 * n_tok * (width + (double) top * ff);
         PI_KT_LAUNCH(PI_KT_MATVEC, PI_BF16, std::min(n_tok, PI_KT_MAXNT - 1), b_up, k_moe_up, dim3((unsigned) ((ff + 3) / 4), (unsigned) (n_tok * top)), dim3(256), 0, s,
                      (const uint16_t *) wup->p0, width, ff, n_exp, x, x_stride, sel_dev, top, exact,
-                     (int) (width % 8 == 0 && ((uintptr_t) wup->p0 % 16) == 0 && ((uintptr_t) x % 16) == 0 && x_stride % 4 == 0), glu, up_dev, pi_abort_word());
+                     (int) (width % 8 == 0 && ((uintptr_t) wup->p0 % 16) == 0 && ((uintptr_t) x % 16) == 0 && x_stride % 4 == 0), glu, limit, up_dev, pi_abort_word());
         PI_CHECK_LAUNCH();
     } else width = out_stride;
     const double b_dn = std::min<double>(n_tok * top, std::max(n_exp, 1)) * 2.0 * ff * width + 4.0 * n_tok * (width + (double) top * ff);
@@ -1090,7 +1167,7 @@ __global__ void __launch_bounds__(256) k_moe_group(const int32_t * __restrict__ 
 
 // acc[j] += W[rows j*16 + (l % 16)][k] * B[slot (l % 16)][k] over K (K % 8 == 0); brow: this lane's B row (nullptr: zeros), wrow[j]: this lane's A rows (nullptr: zeros)
 // glu_off > 0: the B value at k is silu(brow[k]) * brow[glu_off + k] (a gated hidden layer whose two halves were stored raw)
-static __device__ __forceinline__ void hy_mfma_rows(const uint16_t * const wrow[4], const float * brow, int64_t K, int kb, hy_f32x4 acc[4], int64_t glu_off = 0) {
+static __device__ __forceinline__ void hy_mfma_rows(const uint16_t * const wrow[4], const float * brow, int64_t K, int kb, hy_f32x4 acc[4], int64_t glu_off = 0, int glu = PI_GLU_SILU, float limit = 0.0f) {
     for (int64_t k0 = 0; k0 < K; k0 += 32) {
         const int64_t k = k0 + kb * 8;
         const bool k_ok = k < K;
@@ -1102,7 +1179,7 @@ static __device__ __forceinline__ void hy_mfma_rows(const uint16_t * const wrow[
                 const float4 u0 = *(const float4 *) (brow + glu_off + k), u1 = *(const float4 *) (brow + glu_off + k + 4);
                 const float uf[8] = { u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w };
 #pragma unroll
-                for (int i = 0; i < 8; i++) f[i] = f[i] / (1.0f + expf(-f[i])) * uf[i];
+                for (int i = 0; i < 8; i++) f[i] = hy_glu(f[i], uf[i], glu, limit);
             }
 #pragma unroll
             for (int i = 0; i < 8; i++) { const uint32_t u = __float_as_uint(f[i]); b[i] = (uint16_t) ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16); }
@@ -1120,7 +1197,7 @@ static __device__ __forceinline__ void hy_mfma_rows(const uint16_t * const wrow[
 // glu: UP leaves the 2 * ff rows [gate | up] of an expert raw, !UP forms silu(gate) * up while it reads them (bs = 2 * ff, K = ff)
 template <bool UP>
 __global__ void __launch_bounds__(256) k_moe_mfma(const uint16_t * __restrict__ W, int64_t K, int rows, const float * __restrict__ B, int64_t bs, int top, const int32_t * __restrict__ idx,
-                                                  int max_tiles, int glu, float * __restrict__ out, const int32_t * __restrict__ abort_w) {
+                                                  int max_tiles, int glu, float limit, float * __restrict__ out, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 1)) return;
     const int tile = blockIdx.y;
     if (tile >= idx[0]) return;
@@ -1138,7 +1215,7 @@ __global__ void __launch_bounds__(256) k_moe_mfma(const uint16_t * __restrict__ 
     hy_f32x4 acc[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[j] = hy_f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    hy_mfma_rows(wrow, brow, K, kb, acc, !UP && glu ? K : 0);
+    hy_mfma_rows(wrow, brow, K, kb, acc, !UP && glu ? K : 0, glu, limit);
     if (slot < 0) return;
 #pragma unroll
     for (int j = 0; j < 4; j++)
@@ -1180,6 +1257,11 @@ extern "C" int pi_op_moe_experts_grouped(const pi_weight * wup, const pi_weight 
 // glu: w_up holds [gate | up] per expert (2 * ff rows) and up_dev is [n_tok * top][2 * ff]
 extern "C" int pi_op_moe_experts_grouped_act(const pi_weight * wup, const pi_weight * wdown, int n_exp, int ff, int glu, const float * x, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev, int n_tok, int top,
                                              float * up_dev, float * dn_dev, int32_t * idx_dev, float * out, int64_t out_stride, void * stream) {
+    return pi_op_moe_experts_grouped_glu(wup, wdown, n_exp, ff, glu, 0.0f, x, x_stride, sel_dev, selw_dev, n_tok, top, up_dev, dn_dev, idx_dev, out, out_stride, stream);
+}
+extern "C" int pi_op_moe_experts_grouped_glu(const pi_weight * wup, const pi_weight * wdown, int n_exp, int ff, int glu, float limit, const float * x, int64_t x_stride, const int32_t * sel_dev, const float * selw_dev,
+                                             int n_tok, int top, float * up_dev, float * dn_dev, int32_t * idx_dev, float * out, int64_t out_stride, void * stream) {
+    if (glu < PI_GLU_OFF || glu > PI_GLU_CLIPPED) { pi_set_error("pi_op_moe_experts_grouped: hidden layer of kind %d is unknown", glu); return -1; }
     if (!pi_op_moe_grouped_ok(wup, wdown, n_exp, ff, glu, n_tok, top, 0)) { pi_set_error("pi_op_moe_experts_grouped: this shape takes pi_op_moe_experts"); return -1; }
     const int upr = glu ? 2 : 1;
     if (wup->type != PI_BF16 || wdown->type != PI_BF16 || wup->ne1 != (int64_t) n_exp * ff * upr || wdown->ne0 != ff || wdown->ne1 != (int64_t) n_exp * wup->ne0 || x_stride % 4 || ((uintptr_t) x % 16)) {
@@ -1192,10 +1274,10 @@ extern "C" int pi_op_moe_experts_grouped_act(const pi_weight * wup, const pi_wei
     PI_KT_LAUNCH(PI_KT_OTHER, PI_BF16, 1, 8.0 * ns, k_moe_group, dim3(1), dim3(256), 0, s, sel_dev, ns, n_exp, mt, idx_dev, pi_abort_word());
     PI_CHECK_LAUNCH();
     PI_KT_LAUNCH(PI_KT_MMQ, PI_BF16, nta, wbytes + 4.0 * ns * (width + ff), k_moe_mfma<true>, dim3((unsigned) ((ff * upr + 63) / 64), (unsigned) mt), dim3(256), 0, s,
-                 (const uint16_t *) wup->p0, width, ff * upr, x, x_stride, top, idx_dev, mt, glu, up_dev, pi_abort_word());
+                 (const uint16_t *) wup->p0, width, ff * upr, x, x_stride, top, idx_dev, mt, glu, limit, up_dev, pi_abort_word());
     PI_CHECK_LAUNCH();
     PI_KT_LAUNCH(PI_KT_MMQ, PI_BF16, nta, wbytes + 4.0 * ns * (width + ff), k_moe_mfma<false>, dim3((unsigned) ((width + 63) / 64), (unsigned) mt), dim3(256), 0, s,
-                 (const uint16_t *) wdown->p0, (int64_t) ff, (int) width, up_dev, (int64_t) ff * upr, top, idx_dev, mt, glu, dn_dev, pi_abort_word());
+                 (const uint16_t *) wdown->p0, (int64_t) ff, (int) width, up_dev, (int64_t) ff * upr, top, idx_dev, mt, glu, limit, dn_dev, pi_abort_word());
     PI_CHECK_LAUNCH();
     PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 4.0 * n_tok * width * (top + 2), k_moe_combine, dim3((unsigned) ((width + 255) / 256), (unsigned) n_tok), dim3(256), 0, s,
                  dn_dev, width, n_exp, top, x, x_stride, sel_dev, selw_dev, out, out_stride, pi_abort_word());

@@ -32,13 +32,21 @@ static __device__ __forceinline__ float pm_block_sum(float v, float * red) {    
 
 // ---- rotation table: cos / sin of p * base^(-2i / dims), angles formed in double on the host ------------------------------------------------------------
 struct pi_rotary_table { float2 * cs; int n_pos, half; };
-extern "C" void * pi_rotary_table_create(int n_pos, int dims, float base) {
+extern "C" void * pi_rotary_table_create(int n_pos, int dims, float base) { return pi_rotary_table_create_scaled(n_pos, dims, base, 1.0f, 1.0f, 1.0f, 0); }
+// original > 0: long wavelengths are stretched — an angle step whose wavelength 2 pi / f exceeds original / low is divided by `factor`, one below original / high stays, between the two they blend
+extern "C" void * pi_rotary_table_create_scaled(int n_pos, int dims, float base, float factor, float low, float high, int original) {
     if (n_pos < 1 || dims < 0 || (dims & 1)) { pi_set_error("pi_rotary_table_create: %d positions, %d rotated dimensions (an even number)", n_pos, dims); return nullptr; }
+    if (original > 0 && (!(factor > 0.0f) || !(low > 0.0f) || !(high > 0.0f))) { pi_set_error("pi_rotary_table_create: stretching needs positive factor, low and high"); return nullptr; }
     pi_rotary_table * t = new pi_rotary_table{ nullptr, n_pos, dims / 2 };
     if (t->half == 0) return t;
     std::vector<float2> h((size_t) n_pos * t->half);
     for (int i = 0; i < t->half; i++) {
-        const double f = std::pow((double) base, -2.0 * i / dims);
+        double f = std::pow((double) base, -2.0 * i / dims);
+        if (original > 0) {
+            const double wl = 2.0 * M_PI / f, lo_wl = (double) original / high, hi_wl = (double) original / low;
+            if (wl > hi_wl) f /= factor;
+            else if (wl >= lo_wl && high != low) { const double sm = ((double) original / wl - low) / ((double) high - low); f = (1.0 - sm) * f / factor + sm * f; }
+        }
         for (int p = 0; p < n_pos; p++) { const double a = (double) p * f; h[(size_t) p * t->half + i] = make_float2((float) std::cos(a), (float) std::sin(a)); }
     }
     t->cs = (float2 *) pi_malloc(h.size() * sizeof(float2));
@@ -132,6 +140,8 @@ __global__ void __launch_bounds__(64) k_qkv_prepare_any(const float * __restrict
     const float * src = (is_q ? q : k) + (int64_t) t * stride + (int64_t) h * D;
     const float * w = is_q ? qw : kw;
     float * dst = is_q ? q_out + (int64_t) t * qos + (int64_t) h * D : kc + ((int64_t) cell * G + h) * D;
+    const bool none = norm_first == PI_QK_NORM_NONE;
+    norm_first = norm_first == PI_QK_NORM_FIRST;
     float inv1 = 1.0f;
     if (norm_first) {
         float ss = 0.0f;
@@ -151,7 +161,7 @@ __global__ void __launch_bounds__(64) k_qkv_prepare_any(const float * __restrict
         }
         return y;
     };
-    if (norm_first) { for (int i = lane; i < D; i += 64) dst[i] = turned(i); return; }
+    if (norm_first || none) { for (int i = lane; i < D; i += 64) dst[i] = turned(i); return; }
     float ss = 0.0f;
     for (int i = lane; i < D; i += 64) { const float y = turned(i); ss = fmaf(y, y, ss); }
     const float inv = 1.0f / sqrtf(pi_lanes_sum<64>(ss) / (float) D + eps);
@@ -166,7 +176,8 @@ extern "C" int pi_op_qkv_prepare_ex(const float * q, const float * k, const floa
     if (heads < 1 || kv_heads < 1 || heads % kv_heads) { pi_set_error("pi_op_qkv_prepare: %d query heads do not divide over %d key / value heads", heads, kv_heads); return -1; }
     if (!dyn_dev || !cell_pos_dev) { pi_set_error("pi_op_qkv_prepare: the pass's cell table and the cells' position array are required"); return -1; }
     if (pairing != PI_PAIR_HALVES && pairing != PI_PAIR_NEIGHBOURS) { pi_set_error("pi_op_qkv_prepare: pairing %d is unknown", pairing); return -1; }
-    if (norm_first && (!q_norm_w || !k_norm_w)) { pi_set_error("pi_op_qkv_prepare: norm weights are required"); return -1; }
+    if (norm_first < 0 || norm_first > PI_QK_NORM_NONE) { pi_set_error("pi_op_qkv_prepare: norm order %d is unknown", norm_first); return -1; }
+    if (norm_first == PI_QK_NORM_FIRST && (!q_norm_w || !k_norm_w)) { pi_set_error("pi_op_qkv_prepare: norm weights are required"); return -1; }
     PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 8.0 * n_tok * ((double) heads * dim + (double) kv_heads * (dim + vdim)), k_qkv_prepare_any, dim3((unsigned) n_tok, (unsigned) (heads + 2 * kv_heads)), dim3(64), 0, (hipStream_t) stream,
                  q, k, v, stride, q_norm_w, k_norm_w, eps, heads, kv_heads, dim, vdim, rt->cs, rt->half, rt->n_pos, norm_first, pairing, v_norm, pos_dev, q_out, q_out_stride, k_cache, v_cache, cell_pos_dev, dyn_dev, pi_abort_word());
     PI_CHECK_LAUNCH(); return 0;
@@ -223,7 +234,7 @@ template <int RPW>
 __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restrict__ q, int64_t qs, const float * __restrict__ kc, const float * __restrict__ vc, const int32_t * __restrict__ cell_pos,
                                                          const uint32_t * __restrict__ mask, const int32_t * __restrict__ pos, const float * __restrict__ hbias, const float * __restrict__ gate, int64_t gs, int gate_act,
                                                          float scale, float out_mult, int weights, float softcap, int chunk, int H, int G, int D, int V, int n_kv_arg, int tile, int hps, float * __restrict__ out, int64_t os, const int32_t * __restrict__ dyn,
-                                                         const int32_t * __restrict__ abort_w) {
+                                                         const float * __restrict__ sink, int mask_kind, int pool, int pool_off, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 5)) return;
     extern __shared__ float lds[];                // q [hpg][D] | key tile [tile][D + 1], then the value tile [tile][V] in the same place | weights [tile][hpg]
     __shared__ int list[256 * CA_SB], wcnt[4 * CA_SB];
@@ -232,26 +243,30 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
     float * qsh = lds, * ksh = qsh + hpg * D, * wsh = ksh + tile * max(DP, V);
     float * m_run = wsh + tile * hps, * l_run = m_run + hps, * f_run = l_run + hps;        // soft-max weights: per query head the running maximum, denominator, and the factor the sums so far take this tile
     const bool soft = weights != PI_WEIGHTS_SIGMOID;
-    if (soft) for (int m = tid; m < hpg; m += 256) { m_run[m] = weights == PI_WEIGHTS_SOFTMAX_SINK ? 0.0f : -INFINITY; l_run[m] = weights == PI_WEIGHTS_SOFTMAX_SINK ? 1.0f : 0.0f; }      // (a sink: one more key of score 0 that has no value)
+    // (a sink: one more key without a value, of score 0 or of a learned score per head that the scale does not touch)
+    if (soft) for (int m = tid; m < hpg; m += 256) { m_run[m] = sink ? sink[h0 + m] : weights == PI_WEIGHTS_SOFTMAX_SINK ? 0.0f : -INFINITY; l_run[m] = sink || weights == PI_WEIGHTS_SOFTMAX_SINK ? 1.0f : 0.0f; }
     const int n_kv = min(dyn ? dyn[1] : n_kv_arg, n_kv_arg);
     const int words = (n_kv_arg + 31) / 32;
     const uint32_t * mrow = mask + (int64_t) t * words;
     const int p = pos[t];
-    const int first_pos = chunk > 0 ? p / chunk * chunk : 0;
+    // the first position the token sees as itself: the start of its block of `chunk` positions, or of the window of `chunk` positions that ends with the token
+    const int first_pos = chunk <= 0 ? 0 : mask_kind == PI_MASK_WINDOW ? p - chunk + 1 : p / chunk * chunk;
     for (int i = tid; i < hpg * D; i += 256) qsh[i] = q[(int64_t) t * qs + (int64_t) h0 * D + i];
     float acc[CA_MAXOUT];
 #pragma unroll
     for (int i = 0; i < CA_MAXOUT; i++) acc[i] = 0.0f;
     const int n_out = hpg * V;
     for (int c0 = 0; c0 < n_kv; c0 += 256 * CA_SB) {                 // CA_SB blocks of 256 cells at a time: their mask words and positions are loaded together
-        bool vis[CA_SB]; unsigned long long bal[CA_SB];
+        bool vis[CA_SB], far[CA_SB]; unsigned long long bal[CA_SB];
 #pragma unroll
         for (int u = 0; u < CA_SB; u++) {
             const int c = c0 + u * 256 + tid;
             const bool in = c < n_kv;
             const uint32_t word = in ? mrow[c >> 5] : 0u;
             const int cp = in ? cell_pos[c] : -1;
-            vis[u] = in && ((word >> (c & 31)) & 1u) && cp >= first_pos;
+            // behind the window a cell counts where it closes a block of `pool` positions, through the block's pooled row (row pool_off + cell of both caches)
+            far[u] = pool > 0 && cp < first_pos && cp >= 0 && (cp + 1) % pool == 0;
+            vis[u] = in && ((word >> (c & 31)) & 1u) && (cp >= first_pos || far[u]);
         }
 #pragma unroll
         for (int u = 0; u < CA_SB; u++) bal[u] = __ballot(vis[u]);
@@ -267,7 +282,7 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
             for (int w = 0; w < 4; w++) { if (w == wave) mine[u] = total; total += wcnt[u * 4 + w]; }
         if (total == 0) continue;
 #pragma unroll
-        for (int u = 0; u < CA_SB; u++) if (vis[u]) list[mine[u] + __popcll(bal[u] & ((1ull << lane) - 1ull))] = c0 + u * 256 + tid;
+        for (int u = 0; u < CA_SB; u++) if (vis[u]) list[mine[u] + __popcll(bal[u] & ((1ull << lane) - 1ull))] = c0 + u * 256 + tid + (far[u] ? pool_off : 0);
         __syncthreads();
         for (int l0 = 0; l0 < total; l0 += tile) {
             const int nl = min(tile, total - l0);
@@ -330,7 +345,17 @@ extern "C" int pi_op_chunk_attention(const float * q, int64_t q_stride, const fl
 extern "C" int pi_op_chunk_attention_ex(const float * q, int64_t q_stride, const float * k_cache, const float * v_cache, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
                                         const float * head_bias_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int weights, float softcap, int chunk, int heads, int kv_heads,
                                         int dim, int vdim, int n_tok, int n_kv, float * out, int64_t out_stride, const int32_t * dyn_dev, void * stream) {
+    return pi_op_window_attention(q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, nullptr, gate_dev, gate_stride, gate_act, scale, out_mult, weights, softcap, PI_MASK_CHUNK, chunk, 0, 0,
+                                  heads, kv_heads, dim, vdim, n_tok, n_kv, out, out_stride, dyn_dev, stream);
+}
+// the same kernel with the mask kind, pooled far blocks and a learned sink as parameters (`chunk` is the block's or the window's size)
+extern "C" int pi_op_window_attention(const float * q, int64_t q_stride, const float * k_cache, const float * v_cache, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
+                                      const float * head_bias_dev, const float * sink_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int weights, float softcap, int mask_kind, int chunk,
+                                      int pool, int64_t pooled_row_offset, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv, float * out, int64_t out_stride, const int32_t * dyn_dev, void * stream) {
     if (n_tok <= 0) return 0;
+    if (mask_kind != PI_MASK_CHUNK && mask_kind != PI_MASK_WINDOW) { pi_set_error("pi_op_window_attention: mask kind %d is unknown", mask_kind); return -1; }
+    if (pool < 0 || (pool > 0 && (mask_kind != PI_MASK_WINDOW || chunk < 1 || pooled_row_offset < n_kv || pooled_row_offset > 0x3fffffff))) { pi_set_error("pi_op_window_attention: pooled blocks need a window and their rows behind the %d cells", n_kv); return -1; }
+    if (sink_dev && weights == PI_WEIGHTS_SIGMOID) { pi_set_error("pi_op_window_attention: a sink belongs to a soft-max"); return -1; }
     if (weights != PI_WEIGHTS_SIGMOID && weights != PI_WEIGHTS_SOFTMAX && weights != PI_WEIGHTS_SOFTMAX_SINK) { pi_set_error("pi_op_chunk_attention: weights of kind %d are unknown", weights); return -1; }
     if (heads < 1 || kv_heads < 1 || heads % kv_heads || dim < 1 || vdim < 1 || chunk < 0) { pi_set_error("pi_op_chunk_attention: %d query heads over %d key / value heads, sizes %d / %d, chunk %d", heads, kv_heads, dim, vdim, chunk); return -1; }
     int hpg = heads / kv_heads, splits = 1;                            // query heads of a key head that one workgroup serves: all of them, unless their outputs or the LDS plan say otherwise
@@ -341,12 +366,51 @@ extern "C" int pi_op_chunk_attention_ex(const float * q, int64_t q_stride, const
     const size_t lds = lds_of(tile);
     if (hpg * vdim > 256 * CA_MAXOUT || lds > 60 * 1024) { pi_set_error("pi_op_chunk_attention: %d query heads per key head of sizes %d / %d are beyond the kernel (LDS %zu bytes)", hpg, dim, vdim, lds); return -1; }
     const int acct = pi_account_n_kv() > 0 ? pi_account_n_kv() : n_kv;
-    const double visible = chunk > 0 ? std::min(acct, chunk) : acct;
+    const double visible = chunk > 0 ? std::min(acct, chunk) + (pool > 0 ? std::max(acct - chunk, 0) / pool : 0) : acct;
 #define CA_GO(R)     PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), 4.0 * visible * kv_heads * (dim + vdim) + 4.0 * n_tok * heads * (dim + vdim), k_chunk_attention<R>, dim3((unsigned) n_tok, (unsigned) kv_heads, (unsigned) ((heads / kv_heads + hpg - 1) / hpg)), dim3(256), lds, \
                  (hipStream_t) stream, q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, gate_dev, gate_stride, gate_act, scale, out_mult, weights, softcap, chunk, heads, kv_heads, dim, vdim, n_kv, tile, hpg, out, out_stride, \
-                 dyn_dev, pi_abort_word());
+                 dyn_dev, sink_dev, mask_kind, pool, (int) pooled_row_offset, pi_abort_word());
     CA_GO(4);                                                          // (deeper rounds were measured for single tokens: no gain, the registers they take cost as much as the trips they save)
 #undef CA_GO
+    PI_CHECK_LAUNCH(); return 0;
+}
+
+// ---- pooled far blocks: one key / value per block of `pool` positions ------------------------------------------------------------------------------------------
+// grid (token, key / value head).  Only a token that closes a block works: it finds the cells of the block's positions among the cells its mask row shows (its own and the pass's earlier ones
+// included: call this behind the launch that stores the pass's keys and values), sums their rows in position order and leaves the means in row pool_off + its own cell of both caches.
+__global__ void __launch_bounds__(256) k_pool_blocks(float * __restrict__ kc, float * __restrict__ vc, const int32_t * __restrict__ cell_pos, const uint32_t * __restrict__ mask, const int32_t * __restrict__ pos,
+                                                     int pool, int64_t pool_off, int G, int D, int V, int n_kv_arg, const int32_t * __restrict__ dyn, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    extern __shared__ int members[];              // [pool] the cell of every position of the block (-1: none)
+    const int t = blockIdx.x, g = blockIdx.y, tid = threadIdx.x;
+    const int p = pos[t];
+    if ((p + 1) % pool != 0) return;
+    for (int i = tid; i < pool; i += 256) members[i] = -1;
+    __syncthreads();
+    const int n_kv = min(dyn ? dyn[1] : n_kv_arg, n_kv_arg), words = (n_kv_arg + 31) / 32, p0 = p - pool + 1;
+    const uint32_t * mrow = mask + (int64_t) t * words;
+    for (int c = tid; c < n_kv; c += 256) {
+        if (!((mrow[c >> 5] >> (c & 31)) & 1u)) continue;
+        const int cp = cell_pos[c];
+        if (cp >= p0 && cp <= p) members[cp - p0] = c;
+    }
+    __syncthreads();
+    const int64_t own = pool_off + pi_cell_of(dyn, 0, t);
+    for (int i = tid; i < D + V; i += 256) {
+        const bool key = i < D;
+        const float * cache = key ? kc : vc;
+        const int W = key ? D : V, col = key ? i : i - D;
+        float sum = 0.0f;
+        for (int j = 0; j < pool; j++) { const int c = members[j]; if (c >= 0) sum += cache[((int64_t) c * G + g) * W + col]; }
+        (key ? kc : vc)[(own * G + g) * W + col] = sum / (float) pool;
+    }
+}
+extern "C" int pi_op_pool_blocks(float * k_cache, float * v_cache, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev, int pool, int64_t pooled_row_offset, int kv_heads, int dim, int vdim,
+                                 int n_tok, int n_kv, const int32_t * dyn_dev, void * stream) {
+    if (n_tok <= 0) return 0;
+    if (pool < 1 || pool > 8192 || pooled_row_offset < n_kv || kv_heads < 1 || dim < 1 || vdim < 1 || !dyn_dev) { pi_set_error("pi_op_pool_blocks: blocks of %d positions (1..8192), pooled rows from row %lld on behind %d cells", pool, (long long) pooled_row_offset, n_kv); return -1; }
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 4.0 * ((double) n_tok / pool + 1.0) * kv_heads * (dim + vdim) * (pool + 1), k_pool_blocks, dim3((unsigned) n_tok, (unsigned) kv_heads), dim3(256), (size_t) pool * sizeof(int), (hipStream_t) stream,
+                 k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, pool, pooled_row_offset, kv_heads, dim, vdim, n_kv, dyn_dev, pi_abort_word());
     PI_CHECK_LAUNCH(); return 0;
 }
 
