@@ -327,6 +327,10 @@ PI_API int pi_op_copy_rows(const float * src_dev, int64_t src_stride, float * ds
  * (a norm without statistics; alpha_dev: one float on the device).  x_out may be NULL when only the norm is wanted (then a, b, c are still added for h) */
 PI_API int pi_op_sum_tanh_norm(const float * x_dev, int64_t x_stride, const float * a_dev, int64_t a_stride, const float * b_dev, int64_t b_stride, const float * c_dev, int64_t c_stride, int n, int n_tok,
                                float * x_out_dev, int64_t x_out_stride, const float * alpha_dev, const float * w_dev, const float * bias_dev, float * h_out_dev, int64_t h_out_stride, void * stream);
+/* pi_op_sum_tanh_norm and, of its norm output, pi_op_token_shift with one mix: m_out = h + (h_prev - h) * mu; one launch for passes of at most 32 tokens */
+PI_API int pi_op_sum_tanh_norm_shift(const float * x_dev, int64_t x_stride, const float * a_dev, int64_t a_stride, const float * b_dev, int64_t b_stride, const float * c_dev, int64_t c_stride, int n, int n_tok,
+                                     float * x_out_dev, int64_t x_out_stride, const float * alpha_dev, const float * w_dev, const float * bias_dev, float * h_out_dev, int64_t h_out_stride,
+                                     const float * mu_dev, float * state_dev, const int32_t * rec_dev, float * m_out_dev, int64_t m_out_stride, void * stream);
 /* pi_rotary_table_create with angle steps stretched by wavelength l = 2 pi / f against `original` positions: f stays where l < original / high, becomes f / factor where l > original / low, and
  * (1 - s) f / factor + s f with s = (original / l - low) / (high - low) between the two */
 PI_API void * pi_rotary_table_create_scaled(int n_pos, int dims, float base, float factor, float low, float high, int original);
@@ -341,10 +345,11 @@ PI_API int pi_op_pool_blocks(float * k_cache_dev, float * v_cache_dev, const int
                              int n_tok, int n_kv, const int32_t * dyn_dev, void * stream);
 /* pi_op_chunk_attention_ex with the mask kind as a parameter and two more sources of weight.  mask_kind PI_MASK_WINDOW: a token at position p sees the cells of its sequence at positions (p - size, p]
  * (size 0: all up to p); pool > 0 (windows only): and for every block of `pool` positions that ends at or before p - size the pooled row (pi_op_pool_blocks) of the block's last cell, in the same soft-max.
- * sink_dev (nullable, fp32 [heads]; soft-max kinds): exp(sink[h]) joins the denominator, without a value and without the scale (PI_WEIGHTS_SOFTMAX_SINK alone is sink = 0) */
-PI_API int pi_op_window_attention(const float * q_dev, int64_t q_stride, const float * k_cache_dev, const float * v_cache_dev, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
+ * sink_dev (nullable, fp32 [heads]; soft-max kinds): exp(sink[h]) joins the denominator, without a value and without the scale (PI_WEIGHTS_SOFTMAX_SINK alone is sink = 0).
+ * pool_here != 0: an extra slice of workgroups does pi_op_pool_blocks' work in the same launch — allowed where no token of the pass can read a row that the pass writes, n_tok <= size */
+PI_API int pi_op_window_attention(const float * q_dev, int64_t q_stride, float * k_cache_dev, float * v_cache_dev, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
                                   const float * head_bias_dev, const float * sink_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int weights, float softcap, int mask_kind, int size,
-                                  int pool, int64_t pooled_row_offset, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv, float * out_dev, int64_t out_stride, const int32_t * dyn_dev, void * stream);
+                                  int pool, int64_t pooled_row_offset, int pool_here, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv, float * out_dev, int64_t out_stride, const int32_t * dyn_dev, void * stream);
 /* router by logits: z = W x + bias (bias nullable), the `top` largest z win (lowest index on a tie), their weights are the soft-max over the chosen z alone */
 PI_API int pi_op_moe_route_top_logits(const pi_weight * router, const float * bias_dev, const float * x_dev, int64_t x_stride, int n_tok, int top, int exact, int32_t * sel_dev, float * selw_dev, void * stream);
 /* the expert operators with one more kind of hidden layer.  PI_GLU_OFF / PI_GLU_SILU are glu = 0 / 1 of pi_op_moe_experts_act; PI_GLU_CLIPPED: g = min(gate, limit), u = clip(up, -limit, limit)

@@ -132,7 +132,7 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
             ctx->lat_off[i] = lat; lat += (size_t) ctx->n_ctx * H.cell_floats();
             ctx->rec_off[i] = rec; rec += (size_t) ctx->slots->size() * H.state_floats();
             in_w = std::max(in_w, (size_t) std::max(A.in_rows(), std::max(H.mlp == PI_MLP_DENSE_GELU ? H.ff : 0, 3 * H.shared_ff + 1)));
-            att_w = std::max(att_w, (size_t) A.channels() + (size_t) A.heads * A.dim + (size_t) std::max(A.heads * A.vdim, width));
+            att_w = std::max(att_w, (size_t) A.channels() + (size_t) A.heads * A.dim + (size_t) A.heads * A.vdim);
             positions = true;
             if (H.mlp == PI_MLP_MOE_CLIPPED) { up_w = std::max(up_w, (size_t) H.top * 2 * H.ff); sel_w = std::max(sel_w, (size_t) H.top); idx_n = std::max(idx_n, pi_op_moe_grouped_index_ints(nb, H.top, H.n_expert)); }
             continue;
@@ -161,7 +161,7 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
     pi_memset(ctx->lat_cache, 0, std::max<size_t>(lat * 4, 16), nullptr); pi_memset(ctx->rec_state, 0, std::max<size_t>(rec * 4, 16), nullptr);
     if (positions) { if (!(ctx->cell_pos = (int32_t *) dev((size_t) 4 * ctx->n_ctx)) || !(ctx->h_out2 = (float *) dev((size_t) 4 * nb * width)) || !(ctx->ssd_dt = (float *) dev((size_t) 4 * nb * step_w))) return false; pi_memset(ctx->cell_pos, 0, (size_t) 4 * ctx->n_ctx, nullptr); }
     if (hp.depth_average && !(ctx->hist = (float *) dev((size_t) 4 * (hp.hybrid.size() + 1) * nb * width))) return false;
-    if (hp.shared_tanh_norm && (!(ctx->x_pair = (float *) dev((size_t) 4 * nb * 2 * width)) || !(ctx->h_out3 = (float *) dev((size_t) 4 * nb * width)))) return false;
+    if (hp.shared_tanh_norm && (!(ctx->x_pair = (float *) dev((size_t) 4 * nb * 2 * width)) || !(ctx->h_out3 = (float *) dev((size_t) 4 * nb * width)) || !(ctx->nx2 = (float *) dev((size_t) 4 * nb * width)))) return false;
     if (positions && getenv("PI_BRANCH_STREAMS") && !strcmp(getenv("PI_BRANCH_STREAMS"), "1")) {            // (opt-in: measured at 4 % of a token's GPU time at width 2048; by default both branches follow each other on the context's stream)
         if (hipStreamCreateWithFlags(&ctx->branch_stream, hipStreamNonBlocking) != hipSuccess) { err = "hipStreamCreate(branch) failed"; return false; }
         ctx->branch_events.assign(2 * hp.hybrid.size(), nullptr);
@@ -509,10 +509,10 @@ static bool forward_post_norm_blocks(llama_context * ctx, int n_tok, int n_kv) {
 
 // Blocks with ONE tanh norm (hp.shared_tanh_norm), T(y) = tanh(alpha y) * w + b:   h = T(x);  x <- x + mixer(h + (h_prev - h) * shift) + ff(h).   A run of layers may repeat with the same tensors (every
 // entry of hp.hybrid is one run, with a cache and state of its own); in front of a repeated run's first layer x <- W_in [x ; embedding row].
-//   window attention   token shift (+ its state) -> ONE projection [q | k | v (| gate)] -> [convolution per channel (+ its state)] -> q / k norm + rotation (or rotation alone), cache store ->
+//   window attention   ONE projection [q | k | v (| gate)] -> [convolution per channel (+ its state)] -> q / k norm + rotation (or rotation alone), cache store ->
 //                      [pooled rows of the blocks the pass completes] -> soft-max attention over the window (+ pooled far blocks, + a learned sink; * sigmoid(gate) per head) -> W_o
 //   feed-forward       gelu(W_up h) -> W_down;  or router (top logits, soft-max over the chosen) -> clipped gated experts, + the shared expert [gate | up | token gate] -> product -> down
-// A layer ends in ONE row kernel: x + mixer + routed + shared -> x and the NEXT layer's (or the model's last) tanh norm -> h.
+// A layer ends in ONE row kernel: x + mixer + routed + shared -> x, the NEXT layer's tanh norm -> h and its token shift (+ the shifted token's state) -> m; behind the last layer the model's own norm.
 static bool forward_shared_norm_blocks(llama_context * ctx, int n_tok, int n_kv) {
     llama_model * m = ctx->model;
     const pi_hparams & hp = m->hparams;
@@ -520,23 +520,26 @@ static bool forward_shared_norm_blocks(llama_context * ctx, int n_tok, int n_kv)
     const int width = hp.n_embd, ex = ctx->exact, nb = ctx->n_batch, n_slots = ctx->slots->size();
     const float eps = hp.f_norm_rms_eps;
     const size_t n_layer = hp.hybrid.size();
-    float * x = ctx->x, * P = ctx->h_in, * N = ctx->nx, * Y = ctx->h_out, * Y2 = ctx->h_out2, * Y3 = ctx->h_out3, * XP = ctx->x_pair;
+    float * x = ctx->x, * P = ctx->h_in, * N = ctx->nx, * M = ctx->nx2, * Y = ctx->h_out, * Y2 = ctx->h_out2, * Y3 = ctx->h_out3, * XP = ctx->x_pair;
+    // the tanh norm of layer `il` (-> N) and its token-shifted form (-> M, the shifted token's state of that layer's run), behind the sum x + a + b + c -> xo
+    auto norm_shift = [&](size_t il, const float * a, const float * b, const float * c, float * xo) {
+        const pi_hybrid_weights & W = m->hweights[(size_t) hp.hybrid[il].weights];
+        return pi_op_sum_tanh_norm_shift(x, width, a, width, b, width, c, width, width, n_tok, xo, width, W.norm1_alpha, W.norm1, W.norm1_b, N, width, W.mu, ctx->rec_state + ctx->rec_off[il], ctx->rec_dev, M, width, s);
+    };
     bool repeats = false;
     for (const auto & H : hp.hybrid) repeats = repeats || H.loop_entry;
     OP_OK(pi_op_embed(m->tok_embd, ctx->tokens_dev, n_tok, hp.embed_scale, x, s));
     if (repeats) OP_OK(pi_op_copy_rows(x, width, XP + width, 2 * width, width, n_tok, s));                 // the embedding row rides in the second half of [x | x0]
     // x <- W_in [x ; x0] and the entry layer's norm; `sum`: x + a + b + c has not been formed yet
-    auto enter = [&](const pi_hybrid_layer & H, const float * a, const float * b, const float * c) {
-        const pi_hybrid_weights & W = m->hweights[(size_t) H.weights];
+    auto enter = [&](size_t il, const float * a, const float * b, const float * c) {
+        const pi_hybrid_weights & W = m->hweights[(size_t) hp.hybrid[il].weights];
         if (pi_op_sum_tanh_norm(x, width, a, width, b, width, c, width, width, n_tok, XP, 2 * width, nullptr, nullptr, nullptr, nullptr, 0, s) != 0) return false;
         if (pi_op_dense(W.w_loop, XP, 2 * width, n_tok, x, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s) != 0) return false;
-        return pi_op_sum_tanh_norm(x, width, nullptr, 0, nullptr, 0, nullptr, 0, width, n_tok, nullptr, 0, W.norm1_alpha, W.norm1, W.norm1_b, N, width, s) == 0;
+        return norm_shift(il, nullptr, nullptr, nullptr, nullptr) == 0;
     };
     {
-        const pi_hybrid_layer & H0 = hp.hybrid[0];
-        const pi_hybrid_weights & W0 = m->hweights[(size_t) H0.weights];
-        if (H0.loop_entry) { if (!enter(H0, nullptr, nullptr, nullptr)) { ctx->last_error = pi_last_error(); return false; } }
-        else OP_OK(pi_op_sum_tanh_norm(x, width, nullptr, 0, nullptr, 0, nullptr, 0, width, n_tok, nullptr, 0, W0.norm1_alpha, W0.norm1, W0.norm1_b, N, width, s));
+        if (hp.hybrid[0].loop_entry) { if (!enter(0, nullptr, nullptr, nullptr)) { ctx->last_error = pi_last_error(); return false; } }
+        else OP_OK(norm_shift(0, nullptr, nullptr, nullptr, nullptr));
     }
     for (size_t il = 0; il < n_layer; il++) {
         const pi_hybrid_layer & H = hp.hybrid[il];
@@ -544,18 +547,18 @@ static bool forward_shared_norm_blocks(llama_context * ctx, int n_tok, int n_kv)
         if (H.mixer != PI_MIXER_WINDOW_ATTENTION) { ctx->last_error = "blocks with one shared tanh norm are built for the window-attention mixer"; return false; }
         const pi_gate_attention & A = H.left;
         const int64_t pw = A.in_rows(), ch = A.channels(), hd = (int64_t) A.heads * A.dim, hv = (int64_t) A.heads * A.vdim, gd = (int64_t) A.kv_heads * A.dim;
-        float * C = ctx->h_att, * Q = C + (size_t) nb * ch, * O = Q + (size_t) nb * hd, * M = O;       // (the shifted input is done with when the projection has run: the attention's output takes its place)
+        float * C = ctx->h_att, * Q = C + (size_t) nb * ch, * O = Q + (size_t) nb * hd;
         float * kc = ctx->lat_cache + ctx->lat_off[il], * vc = kc + (size_t) A.cell_rows() * ctx->n_ctx * gd;
-        float * shift_state = ctx->rec_state + ctx->rec_off[il], * conv_state = shift_state + (size_t) n_slots * width;
-        OP_OK(pi_op_token_shift(N, width, width, W.mu, 1, shift_state, ctx->rec_dev, n_tok, M, width, s));
+        float * conv_state = ctx->rec_state + ctx->rec_off[il] + (size_t) n_slots * width;         // (behind the run's shifted-token rows)
         OP_OK(pi_op_dense(W.w_in, M, width, n_tok, P, pw, PI_ACT_NONE, pw, PI_ACT_NONE, ex, s));
         const float * qkv = P; int64_t qs = pw;
         if (A.conv > 0) { OP_OK(pi_op_causal_conv(P, pw, (int) ch, A.conv, W.conv_w, nullptr, conv_state, ctx->rec_dev, n_tok, PI_ACT_NONE, C, ch, s)); qkv = C; qs = ch; }
         OP_OK(pi_op_qkv_prepare_ex(qkv, qkv + hd, qkv + hd + gd, qs, W.q_norm, W.k_norm, eps, A.heads, A.kv_heads, A.dim, A.vdim, W.rotary, A.qk_norm, A.pairing, A.v_norm ? 1 : 0, ctx->pos_dev, n_tok, Q, hd, kc, vc,
                                    ctx->cell_pos, ctx->dyn_dev, s));
-        if (A.cell_rows() > 1) OP_OK(pi_op_pool_blocks(kc, vc, ctx->cell_pos, ctx->mask_dev, ctx->pos_dev, A.pool, ctx->n_ctx, A.kv_heads, A.dim, A.vdim, n_tok, n_kv, ctx->dyn_dev, s));
+        const bool pooled = A.cell_rows() > 1, pool_here = pooled && n_tok <= A.chunk;           // (a pass no longer than the window: no token of it reads a pooled row that the pass writes, so the attention launch writes them)
+        if (pooled && !pool_here) OP_OK(pi_op_pool_blocks(kc, vc, ctx->cell_pos, ctx->mask_dev, ctx->pos_dev, A.pool, ctx->n_ctx, A.kv_heads, A.dim, A.vdim, n_tok, n_kv, ctx->dyn_dev, s));
         OP_OK(pi_op_window_attention(Q, hd, kc, vc, ctx->cell_pos, ctx->mask_dev, ctx->pos_dev, nullptr, W.sink, A.gated ? P + ch : nullptr, pw, PI_ACT_SIGMOID, A.scale, 1.0f, A.weights, A.softcap, A.mask_kind, A.chunk,
-                                     A.cell_rows() > 1 ? A.pool : 0, ctx->n_ctx, A.heads, A.kv_heads, A.dim, A.vdim, n_tok, n_kv, O, hv, ctx->dyn_dev, s));
+                                     pooled ? A.pool : 0, ctx->n_ctx, pool_here ? 1 : 0, A.heads, A.kv_heads, A.dim, A.vdim, n_tok, n_kv, O, hv, ctx->dyn_dev, s));
         trace(ctx, "att", (int) il, O, hv, n_tok);
         OP_OK(pi_op_dense(W.w_o, O, hv, n_tok, Y, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
         const float * y2 = nullptr, * y3 = nullptr;
@@ -581,12 +584,12 @@ static bool forward_shared_norm_blocks(llama_context * ctx, int n_tok, int n_kv)
         }
         // the layer's end: the sum, and the norm of what reads the stream next (through the run's input matrix where the next layer opens a repeated run)
         if (il + 1 < n_layer && hp.hybrid[il + 1].loop_entry) {
-            if (!enter(hp.hybrid[il + 1], Y, y2, y3)) { ctx->last_error = pi_last_error(); return false; }
+            if (!enter(il + 1, Y, y2, y3)) { ctx->last_error = pi_last_error(); return false; }
             trace(ctx, "lout", (int) il, XP, width, n_tok, 2 * width);     // (the layer's result went into the first half of [x | x0])
             continue;
         }
-        const pi_hybrid_weights * Wn = il + 1 < n_layer ? &m->hweights[(size_t) hp.hybrid[il + 1].weights] : nullptr;
-        OP_OK(pi_op_sum_tanh_norm(x, width, Y, width, y2, width, y3, width, width, n_tok, x, width, Wn ? Wn->norm1_alpha : m->output_norm_alpha, Wn ? Wn->norm1 : m->output_norm, Wn ? Wn->norm1_b : m->output_norm_b, N, width, s));
+        if (il + 1 < n_layer) OP_OK(norm_shift(il + 1, Y, y2, y3, x));
+        else OP_OK(pi_op_sum_tanh_norm(x, width, Y, width, y2, width, y3, width, width, n_tok, x, width, m->output_norm_alpha, m->output_norm, m->output_norm_b, N, width, s));
         trace(ctx, "lout", (int) il, x, width, n_tok);
     }
     OP_OK(pi_op_dense(m->tok_embd, N, width, n_tok, ctx->logits_dev, hp.n_vocab, PI_ACT_NONE, hp.n_vocab, PI_ACT_NONE, ex, s));

@@ -402,6 +402,48 @@ extern "C" int pi_op_sum_tanh_norm(const float * x, int64_t x_stride, const floa
     PI_CHECK_LAUNCH(); return 0;
 }
 
+// the same with the token shift of the norm's output behind it, m = h + (h_prev - h) * mu (h_prev: the sequence's previous token; pi_op_token_shift's state and slot words), for passes of at most
+// 32 tokens in ONE launch: the thread of a run's first token walks the run for its column with h_prev in a register and leaves the state, so nothing it writes is read by another thread
+#define STN_FRESH (1 << 30)
+#define STN_WALK_MAX_TOKENS 32
+__global__ void __launch_bounds__(256) k_sum_tanh_norm_walk(const float * __restrict__ x, int64_t xs, const float * __restrict__ a, int64_t as, const float * __restrict__ b, int64_t bs, const float * __restrict__ c, int64_t cs,
+                                                            int n, int n_tok, float * __restrict__ xo, int64_t xos, const float * __restrict__ alpha, const float * __restrict__ w, const float * __restrict__ bias,
+                                                            float * __restrict__ ho, int64_t hos, const float * __restrict__ mu, float * __restrict__ state, const int32_t * __restrict__ rec, float * __restrict__ mo,
+                                                            int64_t mos, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.x, i = blockIdx.y * 256 + threadIdx.x;
+    const int word = rec[t], slot = word & ~STN_FRESH;
+    if (i >= n || (t > 0 && (rec[t - 1] & ~STN_FRESH) == slot)) return;
+    const float al = alpha[0], wi = w[i], bi = bias ? bias[i] : 0.0f, mi = mu[i];
+    float prev = (word & STN_FRESH) ? 0.0f : state[(int64_t) slot * n + i];
+    for (int tt = t; tt < n_tok && (rec[tt] & ~STN_FRESH) == slot; tt++) {
+        float v = x[(int64_t) tt * xs + i];
+        if (a) v += a[(int64_t) tt * as + i];
+        if (b) v += b[(int64_t) tt * bs + i];
+        if (c) v += c[(int64_t) tt * cs + i];
+        if (xo) xo[(int64_t) tt * xos + i] = v;
+        const float h = fmaf(tanhf(al * v), wi, bi);
+        ho[(int64_t) tt * hos + i] = h;
+        mo[(int64_t) tt * mos + i] = fmaf(prev - h, mi, h);
+        prev = h;
+    }
+    state[(int64_t) slot * n + i] = prev;
+}
+extern "C" int pi_op_sum_tanh_norm_shift(const float * x, int64_t x_stride, const float * a, int64_t a_stride, const float * b, int64_t b_stride, const float * c, int64_t c_stride, int n, int n_tok,
+                                         float * x_out, int64_t x_out_stride, const float * alpha_dev, const float * w_dev, const float * bias_dev, float * h_out, int64_t h_out_stride,
+                                         const float * mu_dev, float * state_dev, const int32_t * rec_dev, float * m_out, int64_t m_out_stride, void * stream) {
+    if (n_tok <= 0 || n <= 0) return 0;
+    if (!w_dev || !alpha_dev || !h_out || !mu_dev || !state_dev || !rec_dev || !m_out || m_out == h_out) { pi_set_error("pi_op_sum_tanh_norm_shift: the norm, the shift factors, the sequences' state and slot words and two outputs are required"); return -1; }
+    if (n_tok > STN_WALK_MAX_TOKENS) {
+        if (pi_op_sum_tanh_norm(x, x_stride, a, a_stride, b, b_stride, c, c_stride, n, n_tok, x_out, x_out_stride, alpha_dev, w_dev, bias_dev, h_out, h_out_stride, stream) != 0) return -1;
+        return pi_op_token_shift(h_out, h_out_stride, n, mu_dev, 1, state_dev, rec_dev, n_tok, m_out, m_out_stride, stream);
+    }
+    const int rows = 3 + (a != nullptr) + (b != nullptr) + (c != nullptr) + (x_out != nullptr);
+    PI_KT_LAUNCH(PI_KT_OTHER, 0, 1, 4.0 * n * n_tok * rows + 8.0 * n, k_sum_tanh_norm_walk, dim3((unsigned) n_tok, (unsigned) ((n + 255) / 256)), dim3(256), 0, (hipStream_t) stream, x, x_stride, a, a_stride, b, b_stride,
+                 c, c_stride, n, n_tok, x_out, x_out_stride, alpha_dev, w_dev, bias_dev, h_out, h_out_stride, mu_dev, state_dev, rec_dev, m_out, m_out_stride, pi_abort_word());
+    PI_CHECK_LAUNCH(); return 0;
+}
+
 // ---- linear attention with a per-head decay -------------------------------------------------------------------------------------------------------
 // rec[t] = state slot of token t (| 1 << 30 on the first token of a sequence whose state starts from zero), tokens of one slot are consecutive.  Workgroup (head, column block,
 // piece): thread (column j, part sp of R) keeps S[i][j] for its DPT rows i in registers and walks the piece's tokens in order.

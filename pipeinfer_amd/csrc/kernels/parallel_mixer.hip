@@ -30,6 +30,30 @@ static __device__ __forceinline__ float pm_block_sum(float v, float * red) {    
     return s;
 }
 
+// one pooled row: the token at position p = pos[t] closes a block of `pool` positions ((p + 1) % pool == 0, the caller checks): the cells of the block's positions are found among the cells the
+// token's mask row shows, their key / value rows of head g summed in position order, the means left in row pool_off + the token's own cell.  members: `pool` ints of LDS; all 256 threads call
+static __device__ __forceinline__ void pm_pool_block(float * __restrict__ kc, float * __restrict__ vc, const int32_t * __restrict__ cell_pos, const uint32_t * __restrict__ mrow, int p, int pool, int64_t pool_off,
+                                                     int G, int g, int D, int V, int n_kv, int own_cell, int * members) {
+    const int tid = threadIdx.x, p0 = p - pool + 1;
+    for (int i = tid; i < pool; i += 256) members[i] = -1;
+    __syncthreads();
+    for (int c = tid; c < n_kv; c += 256) {
+        if (!((mrow[c >> 5] >> (c & 31)) & 1u)) continue;
+        const int cp = cell_pos[c];
+        if (cp >= p0 && cp <= p) members[cp - p0] = c;
+    }
+    __syncthreads();
+    const int64_t own = pool_off + own_cell;
+    for (int i = tid; i < D + V; i += 256) {
+        const bool key = i < D;
+        const float * cache = key ? kc : vc;
+        const int W = key ? D : V, col = key ? i : i - D;
+        float sum = 0.0f;
+        for (int j = 0; j < pool; j++) { const int c = members[j]; if (c >= 0) sum += cache[((int64_t) c * G + g) * W + col]; }
+        (key ? kc : vc)[(own * G + g) * W + col] = sum / (float) pool;
+    }
+}
+
 // ---- rotation table: cos / sin of p * base^(-2i / dims), angles formed in double on the host ------------------------------------------------------------
 struct pi_rotary_table { float2 * cs; int n_pos, half; };
 extern "C" void * pi_rotary_table_create(int n_pos, int dims, float base) { return pi_rotary_table_create_scaled(n_pos, dims, base, 1.0f, 1.0f, 1.0f, 0); }
@@ -231,12 +255,18 @@ static __device__ __forceinline__ void ca_stage(const float * __restrict__ cache
 #define CA_SB 1                                   // blocks of 256 cells whose visibility is worked out in one round
 #define CA_MAXOUT 16                              // outputs (query head, value column) a thread accumulates: hpg * vdim <= 256 * CA_MAXOUT
 template <int RPW>
-__global__ void __launch_bounds__(256) k_chunk_attention(const float * __restrict__ q, int64_t qs, const float * __restrict__ kc, const float * __restrict__ vc, const int32_t * __restrict__ cell_pos,
+__global__ void __launch_bounds__(256) k_chunk_attention(const float * __restrict__ q, int64_t qs, const float * kc, const float * vc, const int32_t * __restrict__ cell_pos,
                                                          const uint32_t * __restrict__ mask, const int32_t * __restrict__ pos, const float * __restrict__ hbias, const float * __restrict__ gate, int64_t gs, int gate_act,
                                                          float scale, float out_mult, int weights, float softcap, int chunk, int H, int G, int D, int V, int n_kv_arg, int tile, int hps, float * __restrict__ out, int64_t os, const int32_t * __restrict__ dyn,
-                                                         const float * __restrict__ sink, int mask_kind, int pool, int pool_off, const int32_t * __restrict__ abort_w) {
+                                                         const float * __restrict__ sink, int mask_kind, int pool, int pool_off, int pool_z, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 5)) return;
     extern __shared__ float lds[];                // q [hpg][D] | key tile [tile][D + 1], then the value tile [tile][V] in the same place | weights [tile][hpg]
+    if (pool_z > 0 && (int) blockIdx.z == pool_z) {                   // the extra slice of workgroups: the pooled rows of the blocks this pass's tokens close (no token of the pass reads them: the host checked n_tok <= window)
+        const int p = pos[blockIdx.x];
+        if ((p + 1) % pool != 0) return;
+        pm_pool_block((float *) kc, (float *) vc, cell_pos, mask + (int64_t) blockIdx.x * ((n_kv_arg + 31) / 32), p, pool, pool_off, G, blockIdx.y, D, V, min(dyn ? dyn[1] : n_kv_arg, n_kv_arg), pi_cell_of(dyn, 0, blockIdx.x), (int *) lds);
+        return;
+    }
     __shared__ int list[256 * CA_SB], wcnt[4 * CA_SB];
     const int t = blockIdx.x, g = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int hs = blockIdx.z * hps, hpg = min(hps, H / G - hs), h0 = g * (H / G) + hs, DP = D + 1;        // this workgroup's query heads: hpg of them from h0 on (all of the key head's unless they are split over blockIdx.z)
@@ -345,17 +375,18 @@ extern "C" int pi_op_chunk_attention(const float * q, int64_t q_stride, const fl
 extern "C" int pi_op_chunk_attention_ex(const float * q, int64_t q_stride, const float * k_cache, const float * v_cache, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
                                         const float * head_bias_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int weights, float softcap, int chunk, int heads, int kv_heads,
                                         int dim, int vdim, int n_tok, int n_kv, float * out, int64_t out_stride, const int32_t * dyn_dev, void * stream) {
-    return pi_op_window_attention(q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, nullptr, gate_dev, gate_stride, gate_act, scale, out_mult, weights, softcap, PI_MASK_CHUNK, chunk, 0, 0,
+    return pi_op_window_attention(q, q_stride, (float *) k_cache, (float *) v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, nullptr, gate_dev, gate_stride, gate_act, scale, out_mult, weights, softcap, PI_MASK_CHUNK, chunk, 0, 0, 0,
                                   heads, kv_heads, dim, vdim, n_tok, n_kv, out, out_stride, dyn_dev, stream);
 }
 // the same kernel with the mask kind, pooled far blocks and a learned sink as parameters (`chunk` is the block's or the window's size)
-extern "C" int pi_op_window_attention(const float * q, int64_t q_stride, const float * k_cache, const float * v_cache, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
+extern "C" int pi_op_window_attention(const float * q, int64_t q_stride, float * k_cache, float * v_cache, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
                                       const float * head_bias_dev, const float * sink_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int weights, float softcap, int mask_kind, int chunk,
-                                      int pool, int64_t pooled_row_offset, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv, float * out, int64_t out_stride, const int32_t * dyn_dev, void * stream) {
+                                      int pool, int64_t pooled_row_offset, int pool_here, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv, float * out, int64_t out_stride, const int32_t * dyn_dev, void * stream) {
     if (n_tok <= 0) return 0;
     if (mask_kind != PI_MASK_CHUNK && mask_kind != PI_MASK_WINDOW) { pi_set_error("pi_op_window_attention: mask kind %d is unknown", mask_kind); return -1; }
     if (pool < 0 || (pool > 0 && (mask_kind != PI_MASK_WINDOW || chunk < 1 || pooled_row_offset < n_kv || pooled_row_offset > 0x3fffffff))) { pi_set_error("pi_op_window_attention: pooled blocks need a window and their rows behind the %d cells", n_kv); return -1; }
     if (sink_dev && weights == PI_WEIGHTS_SIGMOID) { pi_set_error("pi_op_window_attention: a sink belongs to a soft-max"); return -1; }
+    if (pool_here && (pool < 1 || n_tok > chunk || !dyn_dev)) { pi_set_error("pi_op_window_attention: pooled rows can be written in the same launch only where no token of the pass reads them (%d tokens, window %d)", n_tok, chunk); return -1; }
     if (weights != PI_WEIGHTS_SIGMOID && weights != PI_WEIGHTS_SOFTMAX && weights != PI_WEIGHTS_SOFTMAX_SINK) { pi_set_error("pi_op_chunk_attention: weights of kind %d are unknown", weights); return -1; }
     if (heads < 1 || kv_heads < 1 || heads % kv_heads || dim < 1 || vdim < 1 || chunk < 0) { pi_set_error("pi_op_chunk_attention: %d query heads over %d key / value heads, sizes %d / %d, chunk %d", heads, kv_heads, dim, vdim, chunk); return -1; }
     int hpg = heads / kv_heads, splits = 1;                            // query heads of a key head that one workgroup serves: all of them, unless their outputs or the LDS plan say otherwise
@@ -363,13 +394,14 @@ extern "C" int pi_op_window_attention(const float * q, int64_t q_stride, const f
     int tile = CA_TILE;
     auto lds_of = [&](int tl) { return ((size_t) hpg * dim + (size_t) tl * std::max(dim + 1, vdim) + (size_t) tl * hpg + (size_t) 3 * hpg) * sizeof(float); };
     while (tile > 4 && lds_of(tile) > 60 * 1024) tile >>= 1;
-    const size_t lds = lds_of(tile);
+    const size_t lds = std::max(lds_of(tile), pool_here ? (size_t) pool * sizeof(int) : (size_t) 0);
+    const int n_z = (heads / kv_heads + hpg - 1) / hpg;
     if (hpg * vdim > 256 * CA_MAXOUT || lds > 60 * 1024) { pi_set_error("pi_op_chunk_attention: %d query heads per key head of sizes %d / %d are beyond the kernel (LDS %zu bytes)", hpg, dim, vdim, lds); return -1; }
     const int acct = pi_account_n_kv() > 0 ? pi_account_n_kv() : n_kv;
     const double visible = chunk > 0 ? std::min(acct, chunk) + (pool > 0 ? std::max(acct - chunk, 0) / pool : 0) : acct;
-#define CA_GO(R)     PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), 4.0 * visible * kv_heads * (dim + vdim) + 4.0 * n_tok * heads * (dim + vdim), k_chunk_attention<R>, dim3((unsigned) n_tok, (unsigned) kv_heads, (unsigned) ((heads / kv_heads + hpg - 1) / hpg)), dim3(256), lds, \
+#define CA_GO(R)     PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), 4.0 * visible * kv_heads * (dim + vdim) + 4.0 * n_tok * heads * (dim + vdim), k_chunk_attention<R>, dim3((unsigned) n_tok, (unsigned) kv_heads, (unsigned) (n_z + (pool_here ? 1 : 0))), dim3(256), lds, \
                  (hipStream_t) stream, q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, gate_dev, gate_stride, gate_act, scale, out_mult, weights, softcap, chunk, heads, kv_heads, dim, vdim, n_kv, tile, hpg, out, out_stride, \
-                 dyn_dev, sink_dev, mask_kind, pool, (int) pooled_row_offset, pi_abort_word());
+                 dyn_dev, sink_dev, mask_kind, pool, (int) pooled_row_offset, pool_here ? n_z : 0, pi_abort_word());
     CA_GO(4);                                                          // (deeper rounds were measured for single tokens: no gain, the registers they take cost as much as the trips they save)
 #undef CA_GO
     PI_CHECK_LAUNCH(); return 0;
@@ -382,28 +414,11 @@ __global__ void __launch_bounds__(256) k_pool_blocks(float * __restrict__ kc, fl
                                                      int pool, int64_t pool_off, int G, int D, int V, int n_kv_arg, const int32_t * __restrict__ dyn, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w)) return;
     extern __shared__ int members[];              // [pool] the cell of every position of the block (-1: none)
-    const int t = blockIdx.x, g = blockIdx.y, tid = threadIdx.x;
+    const int t = blockIdx.x, g = blockIdx.y;
     const int p = pos[t];
     if ((p + 1) % pool != 0) return;
-    for (int i = tid; i < pool; i += 256) members[i] = -1;
-    __syncthreads();
-    const int n_kv = min(dyn ? dyn[1] : n_kv_arg, n_kv_arg), words = (n_kv_arg + 31) / 32, p0 = p - pool + 1;
-    const uint32_t * mrow = mask + (int64_t) t * words;
-    for (int c = tid; c < n_kv; c += 256) {
-        if (!((mrow[c >> 5] >> (c & 31)) & 1u)) continue;
-        const int cp = cell_pos[c];
-        if (cp >= p0 && cp <= p) members[cp - p0] = c;
-    }
-    __syncthreads();
-    const int64_t own = pool_off + pi_cell_of(dyn, 0, t);
-    for (int i = tid; i < D + V; i += 256) {
-        const bool key = i < D;
-        const float * cache = key ? kc : vc;
-        const int W = key ? D : V, col = key ? i : i - D;
-        float sum = 0.0f;
-        for (int j = 0; j < pool; j++) { const int c = members[j]; if (c >= 0) sum += cache[((int64_t) c * G + g) * W + col]; }
-        (key ? kc : vc)[(own * G + g) * W + col] = sum / (float) pool;
-    }
+    const int n_kv = min(dyn ? dyn[1] : n_kv_arg, n_kv_arg), words = (n_kv_arg + 31) / 32;
+    pm_pool_block(kc, vc, cell_pos, mask + (int64_t) t * words, p, pool, pool_off, G, g, D, V, n_kv, pi_cell_of(dyn, 0, t), members);
 }
 extern "C" int pi_op_pool_blocks(float * k_cache, float * v_cache, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev, int pool, int64_t pooled_row_offset, int kv_heads, int dim, int vdim,
                                  int n_tok, int n_kv, const int32_t * dyn_dev, void * stream) {

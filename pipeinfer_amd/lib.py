@@ -183,3 +183,15 @@ def _declare(lib):
     lib.pi_op_head_norm_gate.argtypes = [vp, i64, i32, i32, vp, i32, vp, i64, i32, f32, i32, vp, i64, vp]
     lib.pi_op_qkv_prepare_ex.argtypes = [vp, vp, vp, i64, vp, vp, f32, i32, i32, i32, i32, vp, i32, i32, i32, vp, i32, vp, i64, vp, vp, vp, vp, vp]
     lib.pi_op_chunk_attention_ex.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, i64, i32, f32, f32, i32, f32, i32, i32, i32, i32, i32, i32, i32, vp, i64, vp, vp]
+    # layers with one tanh norm, sliding-window attention with pooled far blocks, clipped gated experts
+    lib.pi_op_copy_rows.argtypes = [vp, i64, vp, i64, i32, i32, vp]
+    lib.pi_op_sum_tanh_norm.argtypes = [vp, i64, vp, i64, vp, i64, vp, i64, i32, i32, vp, i64, vp, vp, vp, vp, i64, vp]
+    lib.pi_op_sum_tanh_norm_shift.argtypes = [vp, i64, vp, i64, vp, i64, vp, i64, i32, i32, vp, i64, vp, vp, vp, vp, i64, vp, vp, vp, vp, i64, vp]
+    lib.pi_rotary_table_create_scaled.restype = vp
+    lib.pi_rotary_table_create_scaled.argtypes = [i32, i32, f32, f32, f32, f32, i32]
+    lib.pi_op_pool_blocks.argtypes = [vp, vp, vp, vp, vp, i32, i64, i32, i32, i32, i32, i32, vp, vp]
+    lib.pi_op_window_attention.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, vp, i64, i32, f32, f32, i32, f32, i32, i32, i32, i64, i32, i32, i32, i32, i32, i32, i32, vp, i64, vp, vp]
+    lib.pi_op_moe_route_top_logits.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp, vp, vp]
+    lib.pi_op_moe_experts_glu.argtypes = [vp, vp, i32, i32, i32, f32, vp, i64, vp, vp, i32, i32, i32, vp, vp, i64, vp]
+    lib.pi_op_moe_experts_grouped_glu.argtypes = [vp, vp, i32, i32, i32, f32, vp, i64, vp, vp, i32, i32, vp, vp, vp, vp, i64, vp]
+    lib.pi_op_glu_mul_ex.argtypes = [vp, i64, i32, i32, f32, i64, i32, vp, i64, vp]
