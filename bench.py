@@ -496,7 +496,13 @@ def main():
     ap.add_argument("--compare-postnorm", nargs="?", const="w1024,w2048,w4096", default=None, metavar="SIZES",
                     help="instead of the default workload: the same measurements for the Rafusun design (delta-rule and attention + time-mix layers, the norm after the sum) beside the Vikarax design "
                          "with a dense feed-forward at equal sizes; one JSON line per size")
+    ap.add_argument("--compare-window", nargs="?", const="w1024,w2048,w4096", default=None, metavar="SIZES",
+                    help="instead of the default workload: the same measurements for the Rarevik design (one tanh norm per layer, sliding-window attention with pooled far blocks, clipped routed experts) "
+                         "beside the Vikarax design at equal sizes; one JSON line per size")
     args = ap.parse_args()
+    if args.compare_window:
+        from pipeinfer_amd.tools import hybrid_bench
+        return hybrid_bench.main_window(args.compare_window.split(","), args.cache)
     if args.compare_postnorm:
         from pipeinfer_amd.tools import hybrid_bench
         return hybrid_bench.main_postnorm(args.compare_postnorm.split(","), args.cache)

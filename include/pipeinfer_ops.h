@@ -349,7 +349,10 @@ PI_API int pi_op_pool_blocks(float * k_cache_dev, float * v_cache_dev, const int
  * pool_here != 0: an extra slice of workgroups does pi_op_pool_blocks' work in the same launch — allowed where no token of the pass can read a row that the pass writes, n_tok <= size */
 PI_API int pi_op_window_attention(const float * q_dev, int64_t q_stride, float * k_cache_dev, float * v_cache_dev, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
                                   const float * head_bias_dev, const float * sink_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int weights, float softcap, int mask_kind, int size,
-                                  int pool, int64_t pooled_row_offset, int pool_here, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv, float * out_dev, int64_t out_stride, const int32_t * dyn_dev, void * stream);
+                                  int pool, int64_t pooled_row_offset, int pool_here, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv, float * scratch_dev, size_t scratch_floats, float * out_dev, int64_t out_stride,
+                                  const int32_t * dyn_dev, void * stream);
+/* scratch_dev (nullable): with pi_op_window_attention_scratch_floats(heads, vdim, n_tok) floats a pass of few tokens cuts the cell range into splits that run side by side and merges them in a second launch */
+PI_API size_t pi_op_window_attention_scratch_floats(int heads, int vdim, int n_tok);
 /* router by logits: z = W x + bias (bias nullable), the `top` largest z win (lowest index on a tie), their weights are the soft-max over the chosen z alone */
 PI_API int pi_op_moe_route_top_logits(const pi_weight * router, const float * bias_dev, const float * x_dev, int64_t x_stride, int n_tok, int top, int exact, int32_t * sel_dev, float * selw_dev, void * stream);
 /* the expert operators with one more kind of hidden layer.  PI_GLU_OFF / PI_GLU_SILU are glu = 0 / 1 of pi_op_moe_experts_act; PI_GLU_CLIPPED: g = min(gate, limit), u = clip(up, -limit, limit)

@@ -134,6 +134,7 @@ static bool context_prepare_hybrid(llama_context * ctx, std::string & err) {
             in_w = std::max(in_w, (size_t) std::max(A.in_rows(), std::max(H.mlp == PI_MLP_DENSE_GELU ? H.ff : 0, 3 * H.shared_ff + 1)));
             att_w = std::max(att_w, (size_t) A.channels() + (size_t) A.heads * A.dim + (size_t) A.heads * A.vdim);
             positions = true;
+            ctx->lat_scratch_floats = std::max(ctx->lat_scratch_floats, pi_op_window_attention_scratch_floats(A.heads, A.vdim, nb));
             if (H.mlp == PI_MLP_MOE_CLIPPED) { up_w = std::max(up_w, (size_t) H.top * 2 * H.ff); sel_w = std::max(sel_w, (size_t) H.top); idx_n = std::max(idx_n, pi_op_moe_grouped_index_ints(nb, H.top, H.n_expert)); }
             continue;
         }
@@ -558,7 +559,7 @@ static bool forward_shared_norm_blocks(llama_context * ctx, int n_tok, int n_kv)
         const bool pooled = A.cell_rows() > 1, pool_here = pooled && n_tok <= A.chunk;           // (a pass no longer than the window: no token of it reads a pooled row that the pass writes, so the attention launch writes them)
         if (pooled && !pool_here) OP_OK(pi_op_pool_blocks(kc, vc, ctx->cell_pos, ctx->mask_dev, ctx->pos_dev, A.pool, ctx->n_ctx, A.kv_heads, A.dim, A.vdim, n_tok, n_kv, ctx->dyn_dev, s));
         OP_OK(pi_op_window_attention(Q, hd, kc, vc, ctx->cell_pos, ctx->mask_dev, ctx->pos_dev, nullptr, W.sink, A.gated ? P + ch : nullptr, pw, PI_ACT_SIGMOID, A.scale, 1.0f, A.weights, A.softcap, A.mask_kind, A.chunk,
-                                     pooled ? A.pool : 0, ctx->n_ctx, pool_here ? 1 : 0, A.heads, A.kv_heads, A.dim, A.vdim, n_tok, n_kv, O, hv, ctx->dyn_dev, s));
+                                     pooled ? A.pool : 0, ctx->n_ctx, pool_here ? 1 : 0, A.heads, A.kv_heads, A.dim, A.vdim, n_tok, n_kv, ctx->lat_scratch, ctx->lat_scratch_floats, O, hv, ctx->dyn_dev, s));
         trace(ctx, "att", (int) il, O, hv, n_tok);
         OP_OK(pi_op_dense(W.w_o, O, hv, n_tok, Y, width, PI_ACT_NONE, width, PI_ACT_NONE, ex, s));
         const float * y2 = nullptr, * y3 = nullptr;

@@ -258,7 +258,7 @@ template <int RPW>
 __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restrict__ q, int64_t qs, const float * kc, const float * vc, const int32_t * __restrict__ cell_pos,
                                                          const uint32_t * __restrict__ mask, const int32_t * __restrict__ pos, const float * __restrict__ hbias, const float * __restrict__ gate, int64_t gs, int gate_act,
                                                          float scale, float out_mult, int weights, float softcap, int chunk, int H, int G, int D, int V, int n_kv_arg, int tile, int hps, float * __restrict__ out, int64_t os, const int32_t * __restrict__ dyn,
-                                                         const float * __restrict__ sink, int mask_kind, int pool, int pool_off, int pool_z, const int32_t * __restrict__ abort_w) {
+                                                         const float * __restrict__ sink, int mask_kind, int pool, int pool_off, int pool_z, int n_hz, int n_cs, int split_cells, float * __restrict__ part, const int32_t * __restrict__ abort_w) {
     if (pi_aborted(abort_w, 5)) return;
     extern __shared__ float lds[];                // q [hpg][D] | key tile [tile][D + 1], then the value tile [tile][V] in the same place | weights [tile][hpg]
     if (pool_z > 0 && (int) blockIdx.z == pool_z) {                   // the extra slice of workgroups: the pooled rows of the blocks this pass's tokens close (no token of the pass reads them: the host checked n_tok <= window)
@@ -269,12 +269,18 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
     }
     __shared__ int list[256 * CA_SB], wcnt[4 * CA_SB];
     const int t = blockIdx.x, g = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int hs = blockIdx.z * hps, hpg = min(hps, H / G - hs), h0 = g * (H / G) + hs, DP = D + 1;        // this workgroup's query heads: hpg of them from h0 on (all of the key head's unless they are split over blockIdx.z)
+    // blockIdx.z = head split + n_hz * cell split.  split_cells > 0 (soft-max kinds, few tokens): this workgroup looks at the cells [cs * split_cells, (cs + 1) * split_cells) only and leaves its running
+    // maximum, denominator and un-normalised sums in `part` for k_attention_combine: a single token's tiles then run side by side instead of one after the other
+    const int hz = (int) blockIdx.z % n_hz, cs = (int) blockIdx.z / n_hz;
+    const int hs = hz * hps, hpg = min(hps, H / G - hs), h0 = g * (H / G) + hs, DP = D + 1;        // this workgroup's query heads: hpg of them from h0 on (all of the key head's unless they are split over blockIdx.z)
     float * qsh = lds, * ksh = qsh + hpg * D, * wsh = ksh + tile * max(DP, V);
     float * m_run = wsh + tile * hps, * l_run = m_run + hps, * f_run = l_run + hps;        // soft-max weights: per query head the running maximum, denominator, and the factor the sums so far take this tile
     const bool soft = weights != PI_WEIGHTS_SIGMOID;
     // (a sink: one more key without a value, of score 0 or of a learned score per head that the scale does not touch)
-    if (soft) for (int m = tid; m < hpg; m += 256) { m_run[m] = sink ? sink[h0 + m] : weights == PI_WEIGHTS_SOFTMAX_SINK ? 0.0f : -INFINITY; l_run[m] = sink || weights == PI_WEIGHTS_SOFTMAX_SINK ? 1.0f : 0.0f; }
+    if (soft) for (int m = tid; m < hpg; m += 256) {
+        const bool has_sink = split_cells == 0 && (sink || weights == PI_WEIGHTS_SOFTMAX_SINK);           // (with cell splits the sink joins in the combine)
+        m_run[m] = has_sink ? (sink ? sink[h0 + m] : 0.0f) : -INFINITY; l_run[m] = has_sink ? 1.0f : 0.0f;
+    }
     const int n_kv = min(dyn ? dyn[1] : n_kv_arg, n_kv_arg);
     const int words = (n_kv_arg + 31) / 32;
     const uint32_t * mrow = mask + (int64_t) t * words;
@@ -286,12 +292,13 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
 #pragma unroll
     for (int i = 0; i < CA_MAXOUT; i++) acc[i] = 0.0f;
     const int n_out = hpg * V;
-    for (int c0 = 0; c0 < n_kv; c0 += 256 * CA_SB) {                 // CA_SB blocks of 256 cells at a time: their mask words and positions are loaded together
+    const int c_first = split_cells > 0 ? cs * split_cells : 0, c_end = split_cells > 0 ? min(n_kv, c_first + split_cells) : n_kv;
+    for (int c0 = c_first; c0 < c_end; c0 += 256 * CA_SB) {          // CA_SB blocks of 256 cells at a time: their mask words and positions are loaded together
         bool vis[CA_SB], far[CA_SB]; unsigned long long bal[CA_SB];
 #pragma unroll
         for (int u = 0; u < CA_SB; u++) {
             const int c = c0 + u * 256 + tid;
-            const bool in = c < n_kv;
+            const bool in = c < c_end;
             const uint32_t word = in ? mrow[c >> 5] : 0u;
             const int cp = in ? cell_pos[c] : -1;
             // behind the window a cell counts where it closes a block of `pool` positions, through the block's pooled row (row pool_off + cell of both caches)
@@ -353,6 +360,16 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
             }
         }
     }
+    if (split_cells > 0) {                                            // this split's share: [V sums | maximum | denominator] per (token, head, split)
+        __syncthreads();
+#pragma unroll
+        for (int oi = 0; oi < CA_MAXOUT; oi++) {
+            const int o = oi * 256 + tid;
+            if (o < n_out) { const int m = o / V; part[(((int64_t) t * H + h0 + m) * n_cs + cs) * (V + 2) + o % V] = acc[oi]; }
+        }
+        for (int m = tid; m < hpg; m += 256) { float * pr = part + (((int64_t) t * H + h0 + m) * n_cs + cs) * (V + 2) + V; pr[0] = m_run[m]; pr[1] = l_run[m]; }
+        return;
+    }
 #pragma unroll
     for (int oi = 0; oi < CA_MAXOUT; oi++) {
         const int o = oi * 256 + tid;
@@ -366,6 +383,36 @@ __global__ void __launch_bounds__(256) k_chunk_attention(const float * __restric
     }
 }
 
+// the cell splits of a token's head merged: M = max(maxima, sink), out = sum_s e^(m_s - M) sums_s / (e^(sink - M) + sum_s e^(m_s - M) l_s), in split order; grid (token, head)
+__global__ void __launch_bounds__(128) k_attention_combine(const float * __restrict__ part, int n_cs, int H, int V, const float * __restrict__ sink, int weights, const float * __restrict__ gate, int64_t gs, int gate_act,
+                                                           float out_mult, float * __restrict__ out, int64_t os, const int32_t * __restrict__ abort_w) {
+    if (pi_aborted(abort_w)) return;
+    const int t = blockIdx.x, h = blockIdx.y;
+    const float * pr = part + ((int64_t) t * H + h) * n_cs * (V + 2);
+    const bool has_sink = sink || weights == PI_WEIGHTS_SOFTMAX_SINK;
+    const float sk = sink ? sink[h] : 0.0f;
+    float M = has_sink ? sk : -INFINITY;
+    for (int s = 0; s < n_cs; s++) M = fmaxf(M, pr[(int64_t) s * (V + 2) + V]);
+    float den = has_sink ? expf(sk - M) : 0.0f;
+    for (int s = 0; s < n_cs; s++) { const float ms = pr[(int64_t) s * (V + 2) + V]; if (ms != -INFINITY) den = fmaf(pr[(int64_t) s * (V + 2) + V + 1], expf(ms - M), den); }
+    float gt = gate ? gate[(int64_t) t * gs + h] : 1.0f;
+    if (gate && gate_act == PI_ACT_SIGMOID) gt = pm_sigmoid(gt);
+    for (int v = threadIdx.x; v < V; v += 128) {
+        float a = 0.0f;
+        for (int s = 0; s < n_cs; s++) { const float ms = pr[(int64_t) s * (V + 2) + V]; if (ms != -INFINITY) a = fmaf(pr[(int64_t) s * (V + 2) + v], expf(ms - M), a); }
+        out[(int64_t) t * os + (int64_t) h * V + v] = (den > 0.0f ? a / den : 0.0f) * gt * out_mult;
+    }
+}
+// cell splits of a pass of n_tok tokens over n_kv cells: how many, and the floats of scratch they need (0 splits: the pass is wide enough to fill the device by itself)
+#define CA_SPLIT_MAX 32
+static int ca_cell_splits(int n_tok, int kv_heads, int n_hz, int n_kv, int * split_cells) {
+    if ((int64_t) n_tok * kv_heads * n_hz > 64 || n_kv <= 64) return 0;
+    const int n_cs = std::min(CA_SPLIT_MAX, (n_kv + 63) / 64);
+    *split_cells = ((n_kv + n_cs - 1) / n_cs + 63) / 64 * 64;
+    return (n_kv + *split_cells - 1) / *split_cells;
+}
+extern "C" size_t pi_op_window_attention_scratch_floats(int heads, int vdim, int n_tok) { return (size_t) std::min(n_tok, 64) * heads * CA_SPLIT_MAX * (vdim + 2); }
+
 extern "C" int pi_op_chunk_attention(const float * q, int64_t q_stride, const float * k_cache, const float * v_cache, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
                                      const float * head_bias_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int chunk, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv,
                                      float * out, int64_t out_stride, const int32_t * dyn_dev, void * stream) {
@@ -376,12 +423,13 @@ extern "C" int pi_op_chunk_attention_ex(const float * q, int64_t q_stride, const
                                         const float * head_bias_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int weights, float softcap, int chunk, int heads, int kv_heads,
                                         int dim, int vdim, int n_tok, int n_kv, float * out, int64_t out_stride, const int32_t * dyn_dev, void * stream) {
     return pi_op_window_attention(q, q_stride, (float *) k_cache, (float *) v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, nullptr, gate_dev, gate_stride, gate_act, scale, out_mult, weights, softcap, PI_MASK_CHUNK, chunk, 0, 0, 0,
-                                  heads, kv_heads, dim, vdim, n_tok, n_kv, out, out_stride, dyn_dev, stream);
+                                  heads, kv_heads, dim, vdim, n_tok, n_kv, nullptr, 0, out, out_stride, dyn_dev, stream);
 }
 // the same kernel with the mask kind, pooled far blocks and a learned sink as parameters (`chunk` is the block's or the window's size)
 extern "C" int pi_op_window_attention(const float * q, int64_t q_stride, float * k_cache, float * v_cache, const int32_t * cell_pos_dev, const uint32_t * mask_dev, const int32_t * pos_dev,
                                       const float * head_bias_dev, const float * sink_dev, const float * gate_dev, int64_t gate_stride, int gate_act, float scale, float out_mult, int weights, float softcap, int mask_kind, int chunk,
-                                      int pool, int64_t pooled_row_offset, int pool_here, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv, float * out, int64_t out_stride, const int32_t * dyn_dev, void * stream) {
+                                      int pool, int64_t pooled_row_offset, int pool_here, int heads, int kv_heads, int dim, int vdim, int n_tok, int n_kv, float * scratch, size_t scratch_floats, float * out, int64_t out_stride,
+                                      const int32_t * dyn_dev, void * stream) {
     if (n_tok <= 0) return 0;
     if (mask_kind != PI_MASK_CHUNK && mask_kind != PI_MASK_WINDOW) { pi_set_error("pi_op_window_attention: mask kind %d is unknown", mask_kind); return -1; }
     if (pool < 0 || (pool > 0 && (mask_kind != PI_MASK_WINDOW || chunk < 1 || pooled_row_offset < n_kv || pooled_row_offset > 0x3fffffff))) { pi_set_error("pi_op_window_attention: pooled blocks need a window and their rows behind the %d cells", n_kv); return -1; }
@@ -396,15 +444,24 @@ extern "C" int pi_op_window_attention(const float * q, int64_t q_stride, float *
     while (tile > 4 && lds_of(tile) > 60 * 1024) tile >>= 1;
     const size_t lds = std::max(lds_of(tile), pool_here ? (size_t) pool * sizeof(int) : (size_t) 0);
     const int n_z = (heads / kv_heads + hpg - 1) / hpg;
+    // few tokens and a soft-max: the cell range is cut into splits that run side by side, merged by a second small launch (needs scratch for every split's share)
+    int split_cells = 0, n_cs = weights != PI_WEIGHTS_SIGMOID && scratch ? ca_cell_splits(n_tok, kv_heads, n_z, n_kv, &split_cells) : 0;
+    if (n_cs < 2 || (size_t) n_tok * heads * n_cs * (vdim + 2) > scratch_floats) { n_cs = 1; split_cells = 0; }
     if (hpg * vdim > 256 * CA_MAXOUT || lds > 60 * 1024) { pi_set_error("pi_op_chunk_attention: %d query heads per key head of sizes %d / %d are beyond the kernel (LDS %zu bytes)", hpg, dim, vdim, lds); return -1; }
     const int acct = pi_account_n_kv() > 0 ? pi_account_n_kv() : n_kv;
     const double visible = chunk > 0 ? std::min(acct, chunk) + (pool > 0 ? std::max(acct - chunk, 0) / pool : 0) : acct;
-#define CA_GO(R)     PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), 4.0 * visible * kv_heads * (dim + vdim) + 4.0 * n_tok * heads * (dim + vdim), k_chunk_attention<R>, dim3((unsigned) n_tok, (unsigned) kv_heads, (unsigned) (n_z + (pool_here ? 1 : 0))), dim3(256), lds, \
+#define CA_GO(R)     PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), 4.0 * visible * kv_heads * (dim + vdim) + 4.0 * n_tok * heads * (dim + vdim), k_chunk_attention<R>, dim3((unsigned) n_tok, (unsigned) kv_heads, (unsigned) (n_z * n_cs + (pool_here ? 1 : 0))), dim3(256), lds, \
                  (hipStream_t) stream, q, q_stride, k_cache, v_cache, cell_pos_dev, mask_dev, pos_dev, head_bias_dev, gate_dev, gate_stride, gate_act, scale, out_mult, weights, softcap, chunk, heads, kv_heads, dim, vdim, n_kv, tile, hpg, out, out_stride, \
-                 dyn_dev, sink_dev, mask_kind, pool, (int) pooled_row_offset, pool_here ? n_z : 0, pi_abort_word());
+                 dyn_dev, sink_dev, mask_kind, pool, (int) pooled_row_offset, pool_here ? n_z * n_cs : 0, n_z, n_cs, split_cells, scratch, pi_abort_word());
     CA_GO(4);                                                          // (deeper rounds were measured for single tokens: no gain, the registers they take cost as much as the trips they save)
 #undef CA_GO
-    PI_CHECK_LAUNCH(); return 0;
+    PI_CHECK_LAUNCH();
+    if (split_cells > 0) {
+        PI_KT_LAUNCH(PI_KT_ATT, 0, std::min(n_tok, PI_KT_MAXNT - 1), 4.0 * n_tok * heads * ((double) n_cs * (vdim + 2) + vdim), k_attention_combine, dim3((unsigned) n_tok, (unsigned) heads), dim3(128), 0, (hipStream_t) stream,
+                     scratch, n_cs, heads, vdim, sink_dev, weights, gate_dev, gate_stride, gate_act, out_mult, out, out_stride, pi_abort_word());
+        PI_CHECK_LAUNCH();
+    }
+    return 0;
 }
 
 // ---- pooled far blocks: one key / value per block of `pool` positions ------------------------------------------------------------------------------------------

@@ -190,7 +190,8 @@ def _declare(lib):
     lib.pi_rotary_table_create_scaled.restype = vp
     lib.pi_rotary_table_create_scaled.argtypes = [i32, i32, f32, f32, f32, f32, i32]
     lib.pi_op_pool_blocks.argtypes = [vp, vp, vp, vp, vp, i32, i64, i32, i32, i32, i32, i32, vp, vp]
-    lib.pi_op_window_attention.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, vp, i64, i32, f32, f32, i32, f32, i32, i32, i32, i64, i32, i32, i32, i32, i32, i32, i32, vp, i64, vp, vp]
+    lib.pi_op_window_attention.argtypes = [vp, i64, vp, vp, vp, vp, vp, vp, vp, vp, i64, i32, f32, f32, i32, f32, i32, i32, i32, i64, i32, i32, i32, i32, i32, i32, i32, vp, sz, vp, i64, vp, vp]
+    lib.pi_op_window_attention_scratch_floats.argtypes = [i32, i32, i32]; lib.pi_op_window_attention_scratch_floats.restype = sz
     lib.pi_op_moe_route_top_logits.argtypes = [vp, vp, vp, i64, i32, i32, i32, vp, vp, vp]
     lib.pi_op_moe_experts_glu.argtypes = [vp, vp, i32, i32, i32, f32, vp, i64, vp, vp, i32, i32, i32, vp, vp, i64, vp]
     lib.pi_op_moe_experts_grouped_glu.argtypes = [vp, vp, i32, i32, i32, f32, vp, i64, vp, vp, i32, i32, vp, vp, vp, vp, i64, vp]

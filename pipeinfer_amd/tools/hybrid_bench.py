@@ -7,7 +7,10 @@ same width, depth and head count with Q8_0 weights, the densest quantised type t
 shared one) beside the engine's closest model, which is Fasovik at the same width, depth, head sizes and expert sizes.
 
 `bench.py --compare-postnorm [SIZE,...]`: the Rafusun design (delta-rule layers and attention + time-mix layers in turn, a gated dense feed-forward, the norm after the sum) beside the
-closest model, which is Vikarax at the same width, depth, attention sizes and with a dense feed-forward of the same width."""
+closest model, which is Vikarax at the same width, depth, attention sizes and with a dense feed-forward of the same width.
+
+`bench.py --compare-window [SIZE,...]`: the Rarevik design (one tanh norm per layer, sliding-window attention with pooled far blocks and a sink or with a head gate, clipped routed experts with a
+gated shared one, a repeated run's input matrix) beside the closest model, which is Vikarax at the same width, depth, attention and expert sizes."""
 import ctypes as C
 import json
 import os
@@ -101,7 +104,9 @@ def write_random_tensors(folder, cfg, shapes, ones=(), seed=1):
     with open(os.path.join(folder, "model.safetensors.part"), "wb") as f:
         f.write(struct.pack("<Q", len(h)) + h)
         for name, shp in shapes.items():
-            if len(shp) == 1 or name.endswith(".conv"):
+            if len(shp) == 0:
+                v = np.full((), 0.5, np.float32)
+            elif len(shp) == 1 or name.endswith(".conv"):
                 v = rng.standard_normal(shp, dtype=np.float32) * 0.1 + (1.0 if name.endswith(tuple(ones)) else 0.0)
             else:
                 v = rng.standard_normal(shp, dtype=np.float32) * np.float32(shp[-1] ** -0.5)
@@ -175,6 +180,39 @@ def write_rafusun(folder, size, seed=1):
     cfg = {"architecture": "Rafusun", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "postln_alpha": 2.0, "embedding": {"scale": 1.0, "bigram": {"buckets": 65536, "mul_prev": 8191, "mul_cur": 31}},
            "layers": layers}
     return write_random_tensors(folder, cfg, shapes, ones=("norm", "norm1", "norm2", "ls1", "ls2", ".out"), seed=seed)
+
+
+# Rarevik at the sizes above: pooled block, convolution taps (attention sizes, window = the Vikarax model's chunk, expert sizes as the Vikarax model of the size)
+RAREVIK = {"w1024": (16, 4), "w2048": (16, 4), "w4096": (32, 4)}
+
+
+def write_rarevik(folder, size, seed=1):
+    """layers in turn: window attention with a convolution, pooled far blocks and a sink, then window attention with stretched rotation steps and a head gate; every layer with routed clipped experts
+    and a gated shared one; layers 1 .. 2 are a (once-run) repeated run, so the run's input matrix is part of a pass"""
+    width, n_layer, heads, dim, vdim, _, n_exp, _, top, ff, vocab = SIZES[size]
+    kv_heads, rot, chunk, _, _, _, _, _, _, shared = VIKARAX[size]
+    pool, conv = RAREVIK[size]
+    layers, shapes = [], {"embed": (vocab, width), "loop.in": (width, 2 * width), "final.norm": (width,), "final.norm.b": (width,), "final.norm.alpha": ()}
+    for i in range(n_layer):
+        p, q = "l%d." % i, "l%d.mix." % i
+        mlp = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0}, "router": {"experts": n_exp, "top": top}, "shared": {"ff": shared, "limit": 7.0}}
+        mx = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": dim ** -0.5, "rot": {"dims": rot, "base": 10000.0}, "mask": {"size": chunk}}
+        shapes.update({p + "norm1": (width,), p + "norm1.b": (width,), p + "norm1.alpha": (), p + "shift": (width,),
+                       q + "q": (heads * dim, width), q + "k": (kv_heads * dim, width), q + "v": (kv_heads * vdim, width), q + "o": (width, heads * vdim)})
+        if i % 2 == 0:
+            mx["conv"] = conv
+            mx["mask"]["pool"] = pool
+            shapes.update({q + "q.conv": (heads * dim, conv), q + "k.conv": (kv_heads * dim, conv), q + "v.conv": (kv_heads * vdim, conv), q + "q.norm": (dim,), q + "k.norm": (dim,), q + "sink": (heads,)})
+        else:
+            mx["rot"]["scaling"] = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}
+            shapes[q + "g"] = (heads, width)
+        layers.append({"type": "attention" if i % 2 == 0 else "attention_2", "mixer": mx, "mlp": mlp})
+        shapes.update({p + "mlp.router": (n_exp, width), p + "mlp.router.b": (n_exp,), p + "mlp.shared.sg": (1, width)})
+        for e in ["e%d" % e for e in range(n_exp)] + ["shared"]:
+            f = shared if e == "shared" else ff
+            shapes.update({p + "mlp.%s.gate" % e: (f, width), p + "mlp.%s.up" % e: (f, width), p + "mlp.%s.down" % e: (width, f)})
+    cfg = {"architecture": "Rarevik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "loop": {"start": 1, "stop": min(3, n_layer), "times": 1}, "layers": layers}
+    return write_random_tensors(folder, cfg, shapes, ones=("norm", "norm1"), seed=seed)
 
 
 class KtRow(C.Structure):          # struct pi_kt_row (include/pipeinfer_ops.h)
@@ -287,6 +325,29 @@ def main_postnorm(sizes, cache, n_prompt=512, n_decode=64):
     return 0
 
 
+def main_window(sizes, cache, n_prompt=512, n_decode=64):
+    """Rarevik beside Vikarax (routed experts with a shared one) at equal sizes; one JSON line per size"""
+    lib = L.load()
+    L.check(lib.pi_device_init(0), "pi_device_init")
+    for size in sizes:
+        width, n_layer, heads, dim, vdim, _, n_exp, _, top, ff, vocab = SIZES[size]
+        kv_heads, rot, chunk, r_heads, r_vdim, state, groups, _, _, shared = VIKARAX[size]
+        pool, conv = RAREVIK[size]
+        rar, vik = os.path.join(cache, "rarevik-" + size), os.path.join(cache, "vikarax-" + size)
+        if not os.path.exists(os.path.join(rar, "model.safetensors")):
+            write_rarevik(rar, size)
+        if not os.path.exists(os.path.join(vik, "model.safetensors")):
+            write_vikarax(vik, size)
+        out = {"size": size, "config": {"width": width, "layers": n_layer, "heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "rot_dims": rot, "window": chunk, "pool": pool, "conv": conv,
+                                       "experts": n_exp, "top": top, "ff": ff, "shared_ff": shared, "vikarax_recurrence": {"heads": r_heads, "vdim": r_vdim, "state": state, "groups": groups},
+                                       "vocab": vocab, "n_prompt": n_prompt, "n_decode": n_decode},
+               "rarevik_bf16": measure(lib, rar, n_prompt, n_decode, True),
+               "vikarax_bf16": measure(lib, vik, n_prompt, n_decode, True), "data": "synthetic", "hbm_peak": HBM_PEAK}
+        print(json.dumps(out))
+        sys.stdout.flush()
+    return 0
+
+
 def main(sizes, cache, n_prompt=512, n_decode=64):
     lib = L.load()
     L.check(lib.pi_device_init(0), "pi_device_init")
@@ -315,7 +376,7 @@ def run_phase(design, size, phase, cache, n_prompt=512, n_decode=64):
     L.check(lib.pi_device_init(0), "pi_device_init")
     folder = os.path.join(cache, "%s-%s" % (design, size))
     if not os.path.exists(os.path.join(folder, "model.safetensors")):
-        {"vikarax": write_vikarax, "fasovik": write_fasovik, "rafusun": write_rafusun}[design](folder, size)
+        {"vikarax": write_vikarax, "fasovik": write_fasovik, "rafusun": write_rafusun, "rarevik": write_rarevik}[design](folder, size)
     model = LL.Model(folder)
     ctx = LL.Context(model, n_ctx=n_prompt + n_decode + 64, n_batch=n_prompt)
     ctx.set_precision(False)
@@ -336,7 +397,7 @@ def run_phase(design, size, phase, cache, n_prompt=512, n_decode=64):
 if __name__ == "__main__":
     import argparse
     ap = argparse.ArgumentParser(description="one phase of one folder-described design at one size (for `rocprofv3 --kernel-trace --stats -- python3 -m pipeinfer_amd.tools.hybrid_bench ...`)")
-    ap.add_argument("--design", choices=["vikarax", "fasovik", "rafusun"], required=True)
+    ap.add_argument("--design", choices=["vikarax", "fasovik", "rafusun", "rarevik"], required=True)
     ap.add_argument("--size", choices=sorted(SIZES), default="w2048")
     ap.add_argument("--phase", choices=["prefill", "decode"], required=True)
     ap.add_argument("--cache", default=os.environ.get("PIPEINFER_CACHE", "/tmp/pipeinfer_models"))

@@ -346,8 +346,10 @@ def window_attention_ref(q, kc, vc, cpos, vis, pos, scale, size, pool, sink, gat
 @pytest.mark.parametrize("H,G,D,V,size,pool,n_kv,T", [(1, 1, 4, 6, 3, 2, 20, 2), (3, 1, 8, 6, 7, 3, 70, 5), (8, 2, 80, 72, 48, 16, 700, 9), (4, 4, 33, 130, 100, 0, 300, 4), (12, 2, 16, 24, 0, 0, 520, 3),
                                                        (2, 2, 64, 64, 300, 7, 1100, 2), (4, 2, 96, 64, 9, 64, 400, 6)])
 @pytest.mark.parametrize("kind", ["sink", "gate"])
-def test_window_attention_against_explicit_sums(H, G, D, V, size, pool, n_kv, T, kind):
-    """cells in any order, garbage behind the live cells and in the pooled rows nobody may read, large scores (the running maximum matters); a learned sink, or a plain soft-max with a gate per head"""
+@pytest.mark.parametrize("splits", [False, True])
+def test_window_attention_against_explicit_sums(H, G, D, V, size, pool, n_kv, T, kind, splits):
+    """cells in any order, garbage behind the live cells and in the pooled rows nobody may read, large scores (the running maximum matters); a learned sink, or a plain soft-max with a gate per head;
+    in one launch, and with the cell range cut into splits that a second launch merges (scratch given: passes of few tokens take that path)"""
     U, lib = gpu()
     rng = np.random.default_rng(H + D + n_kv)
     n_ctx = n_kv + 13
@@ -370,8 +372,10 @@ def test_window_attention_against_explicit_sums(H, G, D, V, size, pool, n_kv, T,
     qd, kd, vd, cd, md, pd = U.Dev(q), U.Dev(kc), U.Dev(vc), U.Dev(cpos), U.Dev(pack_mask(vis, n_kv)), U.Dev(pos)
     sd, gd = (U.Dev(sink) if sink is not None else None), (U.Dev(gate) if gate is not None else None)
     od, dyn = U.Dev(nbytes=4 * T * H * V), U.Dev(np.array([0, n_kv, T, 0], np.int32))
+    n_scr = lib.pi_op_window_attention_scratch_floats(H, V, T) if splits else 0
+    scr = U.Dev(np.full(max(n_scr, 1), np.nan, np.float32))
     L.check(lib.pi_op_window_attention(qd.ptr, H * D, kd.ptr, vd.ptr, cd.ptr, md.ptr, pd.ptr, None, sd.ptr if sd else None, gd.ptr if gd else None, H + 2, SIGMOID, 0.6, 1.0, SOFTMAX, 0.0, WINDOW, size,
-                                       pool if size else 0, n_ctx, 0, H, G, D, V, T, n_kv, od.ptr, H * V, dyn.ptr, None))
+                                       pool if size else 0, n_ctx, 0, H, G, D, V, T, n_kv, scr.ptr if splits else None, n_scr, od.ptr, H * V, dyn.ptr, None))
     want = window_attention_ref(q, kc.astype(np.float64), vc.astype(np.float64), cpos, vis, pos, 0.6, size, pool if size else 0, sink, gate[:, :H] if gate is not None else None, H, G, n_ctx)
     assert rel_rms(od.get(np.float32, (T, H, V)), want) < 5e-6
 
@@ -401,8 +405,10 @@ def test_pooled_rows_are_the_means_of_their_blocks(G, D, V, pool, n_tok, here):
     if here:
         H = 2 * G
         q, od = U.Dev(rng.standard_normal((n_tok, H * D)).astype(np.float32)), U.Dev(nbytes=4 * n_tok * H * V)
+        n_scr = lib.pi_op_window_attention_scratch_floats(H, V, n_tok)
+        scr = U.Dev(nbytes=4 * n_scr)                                 # (with scratch: the pooling workgroups sit behind the cell splits' in the launch)
         L.check(lib.pi_op_window_attention(q.ptr, H * D, kd.ptr, vd.ptr, cd.ptr, md.ptr, pd.ptr, None, None, None, 0, NONE, 0.1, 1.0, SOFTMAX, 0.0, WINDOW, max(n_tok, 2), pool, n_ctx, 1, H, G, D, V, n_tok, n_kv,
-                                           od.ptr, H * V, dyn.ptr, None))
+                                           scr.ptr, n_scr, od.ptr, H * V, dyn.ptr, None))
     else:
         L.check(lib.pi_op_pool_blocks(kd.ptr, vd.ptr, cd.ptr, md.ptr, pd.ptr, pool, n_ctx, G, D, V, n_tok, n_kv, dyn.ptr, None))
     got_k, got_v = kd.get(np.float32, (2 * n_ctx, G, D)), vd.get(np.float32, (2 * n_ctx, G, V))
@@ -441,8 +447,10 @@ def test_window_and_block_edges_and_the_sink(size, pool, p):
             k2[n_ctx + b * pool + pool - 1], v2[n_ctx + b * pool + pool - 1] = k2[b * pool:(b + 1) * pool].mean(0), v2[b * pool:(b + 1) * pool].mean(0)
         ds = [U.Dev(a) for a in (q, k2, v2, cpos, pack_mask(vis, n_kv), np.array([p], np.int32), np.array([sink_value], np.float32), np.array([0, n_kv, 1, 0], np.int32))]
         od = U.Dev(nbytes=4 * V)
+        n_scr = lib.pi_op_window_attention_scratch_floats(1, V, 1)
+        scr = U.Dev(nbytes=4 * n_scr)
         L.check(lib.pi_op_window_attention(ds[0].ptr, D, ds[1].ptr, ds[2].ptr, ds[3].ptr, ds[4].ptr, ds[5].ptr, None, ds[6].ptr, None, 0, NONE, 1.0, 1.0, SOFTMAX, 0.0, WINDOW, size, pool, n_ctx, 0, 1, 1, D, V, 1, n_kv,
-                                           od.ptr, V, ds[7].ptr, None))
+                                           scr.ptr, n_scr, od.ptr, V, ds[7].ptr, None))
         return od.get(np.float32, (V,)).astype(np.float64), v2
 
     edge = p - size + 1                                               # the window's first position
@@ -490,8 +498,10 @@ def test_a_far_block_among_hundreds_is_heard():
         vis = np.ones((1, n_kv), bool)
         od = U.Dev(nbytes=4 * 4 * V)
         qd, md, pd, dd = U.Dev(q), U.Dev(pack_mask(vis, n_kv)), U.Dev(np.array([p], np.int32)), U.Dev(np.array([0, n_kv, 1, 0], np.int32))
+        n_scr = lib.pi_op_window_attention_scratch_floats(4, V, 1)
+        scr = U.Dev(nbytes=4 * n_scr)
         L.check(lib.pi_op_window_attention(qd.ptr, 4 * D, kd.ptr, vd.ptr, cd.ptr, md.ptr, pd.ptr, None, None, None, 0, NONE, 1.0, 1.0, SOFTMAX, 0.0, WINDOW, size, pool,
-                                           n_ctx, 0, 4, 2, D, V, 1, n_kv, od.ptr, 4 * V, dd.ptr, None))
+                                           n_ctx, 0, 4, 2, D, V, 1, n_kv, scr.ptr, n_scr, od.ptr, 4 * V, dd.ptr, None))
         got = od.get(np.float32, (4, V))
         mean_v = v2[cell_at[block * pool:(block + 1) * pool], 1].astype(np.float64).mean(0)
         assert np.allclose(got[2], mean_v, atol=1e-5) and np.allclose(got[3], mean_v, atol=1e-5)         # the heads of key head 1
@@ -749,13 +759,13 @@ def test_window_and_block_borders_show_in_prompts_and_in_decoding(tmp_path, exac
     e = Engine(tmp_path, m, n_ctx=340, n_batch=128, exact=exact)
     got = np.concatenate([e.ctx.feed(toks[:290], 0, 0)] + [e.ctx.feed(toks[i:i + 1], i, 0) for i in range(290, 330)])       # every decoded token moves all three windows; blocks close at 293, 299 (and 300, ...)
     assert within(logit_err(got, want), exact)
-    for where, key, value in ((0, "size", 51), (0, "pool", 8), (1, "size", 38), (2, "pool", 31)):
+    for where, key, value in ((0, "size", 51), (0, "pool", 8), (1, "size", 38), (2, "size", 22)):
         if not exact:
             break                                                     # (at serving precision one key more or less among fifty is not far enough from rounding to tell)
         other = json.loads(json.dumps(m["config"]))
         other["layers"][where]["mixer"]["mask"][key] = value
         off = logit_err(got, O.run({"config": other, "tensors": m["tensors"]}, toks))
-        assert np.median(off[100:290]) > 10 * TOL[exact] and np.median(off[290:]) > 10 * TOL[exact], (where, key)
+        assert off[100:290].max() > 30 * TOL[exact] and off[290:].max() > 30 * TOL[exact], (where, key)      # (far away where the one key more or less carries weight, in the prompt and among the decoded tokens)
     e.close()
 
 
